@@ -51,6 +51,8 @@ class NormSpec:
     width: int
     eps: float
     tensors: dict = field(default_factory=dict)  # "weight", "bias"
+    # what is added to the stored weight before it multiplies (a weight stored around zero: 1.0); "rmsnorm" takes it
+    weight_offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -104,7 +106,9 @@ class LatentAttentionSpec:
     """Attention over one compressed row a position: the row c (`rank` wide, normalised) is what the cache
     keeps, and each head's keys (`head_dim` wide) and values (`value_dim` wide) are linear in it. No
     position enters the scores. `window` as in AttentionSpec; `gated`: the heads' outputs are
-    multiplied by the sigmoid of a projection of the mixer's input before the output projection."""
+    multiplied by the sigmoid of a projection of the mixer's input before the output projection
+    (`gate_a_head`: that projection has one row a head, whose sigmoid multiplies the head's whole
+    output). `q_rank` > 0: queries go through a latent of their own, q = Wuq (rmsnorm(Wdq h) * w)."""
 
     kind: str  # "latent_attention"
     width: int
@@ -116,7 +120,9 @@ class LatentAttentionSpec:
     window: int  # 0 = every earlier position
     eps: float  # of the compressed row's norm
     gated: bool = True
-    tensors: dict = field(default_factory=dict)  # q, down, down_norm, up_k, up_v, gate, out
+    tensors: dict = field(default_factory=dict)  # q (or q_down, q_down_norm, q_up), down, down_norm, up_k, up_v, gate, out
+    q_rank: int = 0
+    gate_a_head: bool = False
 
 
 @dataclass(frozen=True)
@@ -257,6 +263,72 @@ class ClampedGLUSpec:
 
 
 @dataclass(frozen=True)
+class DeltaRuleSpec:
+    """A mixer that carries a matrix of state a head and both decays it and takes out of it what its key already holds: with
+    the unit key u = k / sqrt(sum(k^2) + key_eps), a decay w = exp(-decay_scale * sigmoid(W2 tanh(W1 h) + w0)) and a removal
+    rate a = sigmoid(Wa h + ba) a head and key channel, S <- diag(w) S - (a * u)(u^T S) + k v^T (both terms read the old S),
+    o = S^T r; each head's o brought to unit root mean square, times a weight and sigmoid(Wg h), then the output projection."""
+
+    kind: str  # "delta_rule"
+    width: int
+    n_head: int
+    head_dim: int
+    decay_rank: int
+    eps: float
+    decay_scale: float = 0.6065306597126334  # exp(-1/2)
+    key_eps: float = 1e-6
+    tensors: dict = field(default_factory=dict)  # r, k, v, a, a_bias, g, w1, w2, w0, norm, out
+
+
+@dataclass(frozen=True)
+class DifferentialAttentionSpec:
+    """Attention in two maps a head that share their values: queries and keys hold [map 1 | map 2] a head, each map an
+    ordinary softmax attention under the window, and a head's result is o = a1 - lam * a2 with lam = exp(lq1 . lk1) -
+    exp(lq2 . lk2) + lam_init, brought to unit root mean square over the head (no weight) and multiplied by `out_scale`.
+    `conv_taps` > 0: every channel of the projected q, k and v passes a causal convolution over time first, whose last
+    taps - 1 inputs are part of a request's state."""
+
+    kind: str  # "differential_attention"
+    width: int
+    n_head: int
+    n_kv_head: int
+    head_dim: int
+    value_dim: int
+    scale: float
+    window: int  # 0 = every earlier position
+    lam_init: float
+    out_scale: float
+    eps: float
+    conv_taps: int = 0
+    tensors: dict = field(default_factory=dict)  # q, q_bias, k, k_bias, v, v_bias, q_conv, k_conv, v_conv, lq1, lk1, lq2, lk2, out
+
+
+@dataclass(frozen=True)
+class NormedPowersFFNSpec:
+    """A feed-forward whose activation is a learned mix of the first `len(act)` - 1 powers of its input, each brought to unit root
+    mean square over the inner width: down(c_1 N(z) + c_2 N(z^2) + ... + c_last), z = up h, powers entry by entry."""
+
+    kind: str  # "normed_powers_ffn"
+    width: int
+    inner: int
+    eps: float
+    powers: int = 3
+    tensors: dict = field(default_factory=dict)  # up, act [powers + 1], down
+
+
+@dataclass(frozen=True)
+class ReentrySpec:
+    """What happens to the stream ahead of a layer at which a repeated stretch of layers begins a pass: x <- W [x ; x0] + steps[index],
+    x0 being the embedding's output, W [width, 2 width] and `steps` one row a pass."""
+
+    kind: str  # "reentry"
+    width: int
+    index: int
+    passes: int
+    tensors: dict = field(default_factory=dict)  # weight, steps
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One block: which parts it has and how they are arranged.
 
@@ -265,6 +337,9 @@ class LayerSpec:
     arrangement "post_norm_gated": x += norm_mixer(gate_mixer * mixer(conv(x))); x += norm_ffn(gate_ffn *
     ffn(x)): the sublayers read the stream itself, the norms stand on their results; `input_conv`
     (what the mixer reads is first convolved over time) and the gates are optional.
+    arrangement "parallel_pair": x += mixer(c1(norm_mixer(x))) + ffn(c2(norm_ffn(x))): two norms of the same x, each
+    followed by a convolution over time of its own (`input_conv`, `ffn_conv`: h <- h + conv(h); optional).
+    `entry`: what is done to the stream before the layer runs (a spec of the entry registry), or None.
     """
 
     mixer: Any
@@ -275,6 +350,8 @@ class LayerSpec:
     input_conv: Any = None
     gate_mixer: Any = None
     gate_ffn: Any = None
+    ffn_conv: Any = None
+    entry: Any = None
 
 
 @dataclass(frozen=True)
@@ -299,6 +376,7 @@ class HeadSpec:
     vocab_size: int
     logit_scale: float
     tensors: dict = field(default_factory=dict)  # "weight" (may name the embedding table), "bias"
+    softcap: float = 0.0  # > 0: logits <- softcap * tanh(logits / softcap), last of all
 
 
 @dataclass(frozen=True)

@@ -111,6 +111,15 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_gated_group_norm),
     LIYAB_ENTRY(liyab_qk_prepare),
     LIYAB_ENTRY(liyab_attention_scored),
+    LIYAB_ENTRY(liyab_norm_shift),
+    LIYAB_ENTRY(liyab_ring_keep),
+    LIYAB_ENTRY(liyab_normed_powers),
+    LIYAB_ENTRY(liyab_softcap),
+    LIYAB_ENTRY(liyab_delta_prepare),
+    LIYAB_ENTRY(liyab_delta_scan),
+    LIYAB_ENTRY(liyab_head_norm_gate),
+    LIYAB_ENTRY(liyab_maps_store),
+    LIYAB_ENTRY(liyab_maps_join),
 };
 constexpr int kNumEntries = static_cast<int>(sizeof(kEntries) / sizeof(kEntries[0]));
 

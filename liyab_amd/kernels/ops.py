@@ -1597,3 +1597,193 @@ def gate_rows(x: torch.Tensor, gate: torch.Tensor) -> None:
     if gate.dtype != torch.float32 or gate.shape != x.shape:
         raise KernelError("gate_rows: the gate must be float32 and of x's shape")
     _lib.call("liyab_gate_rows", x.data_ptr(), dtype_code(x.dtype), ldx, gate.data_ptr(), ldg, x.shape[0], x.shape[1], _stream())
+
+
+# -- two norms of one stream with a convolution over time each; rings of kept rows; small row kernels ---------
+SHIFT_MAX_TAPS = 16
+
+
+class StateSlice:
+    """A stretch of a layer's per-request state [slots, floats a slot] float32 that one part owns: `offset` floats from a
+    slot's start, `size` floats long. Kernels get the stretch's address in slot 0 and the slots' stride."""
+
+    def __init__(self, state: torch.Tensor, offset: int, size: int):
+        stride = _state(state, "a part's state")
+        if offset < 0 or size < 0 or offset + size > stride:
+            raise KernelError(f"a stretch of {size} floats at {offset} does not lie in a slot of {stride}")
+        self.state, self.offset, self.size = state, int(offset), int(size)
+
+    @property
+    def stride(self) -> int:
+        return self.state.shape[1]
+
+    @property
+    def n_slots(self) -> int:
+        return self.state.shape[0]
+
+    def data_ptr(self) -> int:
+        return self.state.data_ptr() + 4 * self.offset
+
+    def sub(self, offset: int, size: int) -> "StateSlice":
+        if offset < 0 or offset + size > self.size:
+            raise KernelError("a stretch past its owner's")
+        return StateSlice(self.state, self.offset + offset, size)
+
+
+def norm_shift(out: torch.Tensor, x: torch.Tensor, weights: torch.Tensor, offset: float, eps: float, conv: Optional[torch.Tensor],
+               ring: Optional[StateSlice], ctx, hbuf: Optional[torch.Tensor] = None) -> None:
+    """out[s, t] = h_s[t] + sum_j conv[s, :, j] * h_s[t - taps + 1 + j] with h_s = x / sqrt(mean(x^2) + eps) * (weights[s] + offset)
+    over each request's own rows in time (conv None: out = h). x float32 [n, d] (the step's rows), weights float32 [S, d],
+    conv float32 [S, d, taps], out [S, n, d] float32 or bfloat16; rows before the step's portion come from `ring` ((taps - 1) x
+    [S, d] floats, position p at place p % (taps - 1)); `hbuf` float32 [n, S * d] gets h itself, for `ring_keep`."""
+    _dev(out, "out")
+    _dev(x, "x")
+    n, d = x.shape
+    S = weights.shape[0] if weights.dim() == 2 else 0
+    if x.dtype != torch.float32 or not x.is_contiguous() or ctx.n_tokens != n:
+        raise KernelError("norm_shift: x must be the step's contiguous float32 rows")
+    if not 1 <= S <= 2 or tuple(out.shape) != (S, n, d) or not out.is_contiguous():
+        raise KernelError(f"norm_shift: out must be contiguous [{S}, {n}, {d}] for one or two sublayers")
+    _f32vec(weights, "norm weights", S * d)
+    taps = 0
+    if conv is not None:
+        _dev(conv, "conv")
+        if conv.dtype != torch.float32 or conv.dim() != 3 or tuple(conv.shape[:2]) != (S, d) or not conv.is_contiguous():
+            raise KernelError(f"norm_shift: the convolution's weights must be contiguous float32 [{S}, {d}, taps]")
+        taps = conv.shape[2]
+        if not 1 <= taps <= SHIFT_MAX_TAPS:
+            raise KernelError(f"norm_shift: {taps} taps; 1 to {SHIFT_MAX_TAPS} are taken")
+    if taps > 1 and (ring is None or ring.size != (taps - 1) * S * d):
+        raise KernelError(f"norm_shift: {taps} taps need a ring of {(taps - 1) * S * d} floats a slot")
+    if hbuf is not None and (hbuf.dtype != torch.float32 or tuple(hbuf.shape) != (n, S * d) or not hbuf.is_contiguous()):
+        raise KernelError(f"norm_shift: hbuf must be contiguous float32 [{n}, {S * d}]")
+    _step_lists(ctx, n)
+    _lib.call("liyab_norm_shift", out.data_ptr(), dtype_code(out.dtype), _ptr(hbuf), x.data_ptr(), weights.data_ptr(), float(offset), float(eps),
+              _ptr(conv), taps, ring.data_ptr() if taps > 1 else None, ring.stride if taps > 1 else 0, ring.n_slots if taps > 1 else 0,
+              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, d, S, _stream())
+
+
+def ring_keep(ring: StateSlice, places: int, src: torch.Tensor, ctx) -> None:
+    """The last `places` rows of each request in the step go to its history: position p to place p % places of `ring` (places x
+    [width] floats); src float32 [n, width] (columns of wider rows are fine). Rows behind the step's tokens are left out. It
+    runs after every kernel of the step that reads the ring."""
+    ld = _rows(src, "src")
+    n, width = src.shape
+    if src.dtype != torch.float32 or ctx.n_tokens != n or places < 1 or ring.size != places * width:
+        raise KernelError(f"ring_keep: the step's float32 rows of {width} and a ring of {places} places of them are needed")
+    _step_lists(ctx, n)
+    _i32(ctx.context_lens, "context_lens", ctx.n_seqs)
+    _lib.call("liyab_ring_keep", ring.data_ptr(), ring.stride, places, ring.n_slots, src.data_ptr(), ld, width, ctx.tok_seq.data_ptr(),
+              ctx.positions.data_ptr(), ctx.context_lens.data_ptr(), ctx.state_slots.data_ptr(), ctx.seq_starts.data_ptr() + 4 * ctx.n_seqs, n, _stream())
+
+
+def normed_powers(out: torch.Tensor, z: torch.Tensor, coef: torch.Tensor, eps: float) -> None:
+    """out = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3 with N(v) = v / sqrt(mean(v^2) + eps) over a row; z float32 rows [n, ff] (columns
+    of wider rows are fine), coef float32 [4] on the device, out contiguous [n, ff] float32 or bfloat16."""
+    _dev(out, "out")
+    ld = _rows(z, "z")
+    n, ff = z.shape
+    if z.dtype != torch.float32 or tuple(out.shape) != (n, ff) or not out.is_contiguous():
+        raise KernelError("normed_powers: z must be float32 rows and out contiguous of its shape")
+    _f32vec(coef, "the powers' weights", 4)
+    _lib.call("liyab_normed_powers", out.data_ptr(), dtype_code(out.dtype), z.data_ptr(), ld, n, ff, coef.data_ptr(), float(eps), _stream())
+
+
+def softcap_(t: torch.Tensor, cap: float) -> torch.Tensor:
+    """t <- cap * tanh(t / cap) in place; t contiguous float32."""
+    _dev(t, "t")
+    if t.dtype != torch.float32 or not t.is_contiguous() or not cap > 0:
+        raise KernelError("softcap_: a contiguous float32 tensor and a positive cap are needed")
+    _lib.call("liyab_softcap", t.data_ptr(), float(cap), t.numel(), _stream())
+    return t
+
+
+# -- the delta-rule recurrence -------------------------------------------------------------------------------
+def delta_takes(head_dim: int) -> bool:
+    """Whether the delta-rule kernel takes heads of this size (a quarter of a column's rows in a lane's registers)."""
+    return 1 <= head_dim <= 256
+
+
+def delta_rule(out: torch.Tensor, proj: torch.Tensor, wraw: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor, norm_w: Optional[torch.Tensor],
+               eps: float, state: StateSlice, ctx, *, n_head: int, head_dim: int, decay_scale: float, key_eps: float) -> None:
+    """The decayed delta rule over each request's rows of the step. proj float32 [n, >= 5 * H * D] = [r | k | v | removal logits |
+    gate logits | ...], wraw float32 [n, H * D] the decay's logits before w0; with u = k / sqrt(sum(k^2) + key_eps), w = exp(-decay_scale
+    * sigmoid(wraw + w0)), a = sigmoid(removal + a_bias): S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r a head; out [n, H * D]
+    (compute dtype) = o / rms(o over the head) * norm_w * sigmoid(gate). `state`: the heads' matrices [H, D, D] of a slot."""
+    _dev(out, "out")
+    n, HD = out.shape
+    H, D = n_head, head_dim
+    ld, ldw = _rows(proj, "proj"), _rows(wraw, "wraw")
+    if HD != H * D or proj.dtype != torch.float32 or proj.shape[0] != n or proj.shape[1] < 5 * HD or not out.is_contiguous() or ctx.n_tokens != n:
+        raise KernelError(f"delta_rule: needs the step's float32 proj [n, >= {5 * H * D}] and a contiguous out [n, {H * D}]")
+    if wraw.dtype != torch.float32 or tuple(wraw.shape) != (n, HD):
+        raise KernelError(f"delta_rule: the decay's logits must be float32 [{n}, {HD}]")
+    for t, what in ((w0, "w0"), (a_bias, "a_bias"), (norm_w, "norm weight")):
+        _f32vec(t, what, HD)
+    if not delta_takes(D) or state.size != H * D * D:
+        raise KernelError(f"delta_rule: heads of {D} with {state.size} floats of state a slot")
+    _step_lists(ctx, n)
+    ws = ctx.workspace
+    prep = ws.get("delta_prep", (n, 3, HD), torch.float32)
+    o = ws.get("delta_o", (n, HD), torch.float32)
+    p = proj.data_ptr()
+    _lib.call("liyab_delta_prepare", prep.data_ptr(), p + 4 * HD, wraw.data_ptr(), p + 12 * HD, ld, ldw, w0.data_ptr(), a_bias.data_ptr(),
+              float(decay_scale), float(key_eps), n, H, D, _stream())
+    _lib.call("liyab_delta_scan", o.data_ptr(), p, p + 4 * HD, p + 8 * HD, ld, prep.data_ptr(), state.data_ptr(), state.stride, state.n_slots,
+              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, H, D, _stream())
+    _lib.call("liyab_head_norm_gate", out.data_ptr(), dtype_code(out.dtype), o.data_ptr(), p + 16 * HD, ld, _ptr(norm_w), float(eps), n, H, D, _stream())
+
+
+# -- attention in two maps a head --------------------------------------------------------------------------------
+def maps_store(proj: torch.Tensor, q_out: torch.Tensor, k1: torch.Tensor, k2: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor,
+               conv: Optional[torch.Tensor], ring: Optional[StateSlice], ctx, *, n_head: int, n_kv_head: int, head_dim: int, value_dim: int,
+               num_pages: Optional[int] = None) -> None:
+    """From a projection's float32 rows [q | k | v] (a query or key head = [map 1 | map 2]) through a causal convolution over time on
+    each channel (conv float32 [C, taps] or None; rows before the step's portion from `ring`, (taps - 1) x [C] floats) to queries
+    q_out [n, 2, H * P] and keys and values in their slots of the pages (k1, k2, v_cache [pages, G, page_size, P]), zeros behind a
+    head's own entries."""
+    H, G, D, V = n_head, n_kv_head, head_dim, value_dim
+    n = proj.shape[0]
+    ld = _rows(proj, "proj")
+    C = 2 * H * D + 2 * G * D + G * V
+    if proj.dtype != torch.float32 or proj.shape[1] != C or ctx.n_tokens != n:
+        raise KernelError(f"maps_store: the step's float32 rows of {C} channels are needed, got {tuple(proj.shape)} {proj.dtype}")
+    for c in (k1, k2, v_cache):
+        _dev(c, "cache")
+        if c.dim() != 4 or tuple(c.shape) != tuple(k1.shape) or c.shape[1] != G or not c.is_contiguous() or c.dtype != q_out.dtype:
+            raise KernelError("maps_store: the three planes must be contiguous [pages, kv heads, page_size, P] in the queries' dtype")
+    P = k1.shape[3]
+    _dev(q_out, "q_out")
+    if P < max(D, V) or tuple(q_out.shape) != (n, 2, H * P) or not q_out.is_contiguous():
+        raise KernelError(f"maps_store: q_out must be contiguous [{n}, 2, {H * P}]")
+    taps = 0
+    if conv is not None:
+        _dev(conv, "conv")
+        if conv.dtype != torch.float32 or tuple(conv.shape[:1]) != (C,) or conv.dim() != 2 or not conv.is_contiguous():
+            raise KernelError(f"maps_store: the convolution's weights must be contiguous float32 [{C}, taps]")
+        taps = conv.shape[1]
+        if not 1 <= taps <= SHIFT_MAX_TAPS:
+            raise KernelError(f"maps_store: {taps} taps; 1 to {SHIFT_MAX_TAPS} are taken")
+    if taps > 1 and (ring is None or ring.size != (taps - 1) * C):
+        raise KernelError(f"maps_store: {taps} taps need a ring of {(taps - 1) * C} floats a slot")
+    _i32(slots, "slots", n)
+    _step_lists(ctx, n)
+    _lib.call("liyab_maps_store", proj.data_ptr(), ld, _ptr(conv), taps, ring.data_ptr() if taps > 1 else None, ring.stride if taps > 1 else 0,
+              ring.n_slots if taps > 1 else 0, q_out.data_ptr(), k1.data_ptr(), k2.data_ptr(), v_cache.data_ptr(), dtype_code(q_out.dtype),
+              slots.data_ptr(), k1.shape[2], _pages(k1, num_pages), ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(),
+              ctx.state_slots.data_ptr(), n, H, G, D, V, P, _stream())
+
+
+def maps_join(out: torch.Tensor, a1: torch.Tensor, a2: torch.Tensor, lam: float, eps: float, out_scale: float, *, n_head: int, value_dim: int) -> None:
+    """out[t, h] = unit_rms(a1[t, h] - lam * a2[t, h]) * out_scale over a head's first `value_dim` entries; a1, a2 [n, H * P] rows of
+    one stride (two maps of one buffer), out contiguous [n, H * value_dim], all of one dtype."""
+    _dev(out, "out")
+    lda, ldb = _rows(a1, "a1"), _rows(a2, "a2")
+    n, H, V = out.shape[0], n_head, value_dim
+    if a1.shape != a2.shape or lda != ldb or a1.shape[0] != n or a1.shape[1] % H or a1.dtype != out.dtype or a2.dtype != out.dtype:
+        raise KernelError("maps_join: two maps of one shape, stride and dtype are needed")
+    P = a1.shape[1] // H
+    if P < V or tuple(out.shape) != (n, H * V) or not out.is_contiguous():
+        raise KernelError(f"maps_join: out must be contiguous [{n}, {H * V}]")
+    _lib.call("liyab_maps_join", out.data_ptr(), a1.data_ptr(), a2.data_ptr(), lda, dtype_code(out.dtype), float(lam), float(eps), float(out_scale),
+              n, H, V, P, _stream())

@@ -129,11 +129,14 @@ class DecoderModel:
             # what a block may have of its own between the stream and its sublayers (a convolution on a
             # sublayer's input, gates on the results): built here, handed over by name where the plan has them
             extras = {}
-            for name, family in (("input_conv", "conv"), ("gate_mixer", "gate"), ("gate_ffn", "gate")):
+            for name, family in (("input_conv", "conv"), ("ffn_conv", "conv"), ("gate_mixer", "gate"), ("gate_ffn", "gate")):
                 extra = getattr(spec, name, None)
                 if extra is not None:
                     extras[name] = build_part(family, extra, store, dtype)
             self.blocks.append(find_part("block", spec.arrangement)(spec, mixer, ffn, norm_mixer, norm_ffn, **extras))
+        # what is done to the stream ahead of a layer (where a repeated stretch of layers begins a pass), by the layer's number
+        self.entries = {i: build_part("entry", spec.entry, store, dtype) for i, spec in enumerate(plan.layers) if getattr(spec, "entry", None) is not None}
+        self.keeps_embedding = any(getattr(e, "needs_embedding", False) for e in self.entries.values())
         self.final_norm = build_part("norm", plan.final_norm, store, dtype) if plan.final_norm is not None else None
         self.head = build_part("head", plan.head, store, dtype)
         self.order = list(plan.order)
@@ -161,9 +164,9 @@ class DecoderModel:
         # sees all the step's rows says that it takes them (`takes_padding_rows`): the embedding, a position
         # encoding of the stream, and every block with its mixer, feed-forward and norms. The final norm and
         # the head see the wanted rows only.
-        every = [self.embedding, self.residual_position]
+        every = [self.embedding, self.residual_position] + list(self.entries.values())
         for block in self.blocks:
-            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn", "conv", "gate_mixer", "gate_ffn")]
+            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn", "conv", "ffn_conv", "gate_mixer", "gate_ffn")]
         self.takes_padding_rows = all(bool(getattr(part, "takes_padding_rows", False)) for part in every if part is not None)
 
     # -- what the cache manager needs to know ---------------------------------
@@ -204,10 +207,21 @@ class DecoderModel:
         self.embedding.forward(ctx, x, position_table=fused)
         if self.residual_position is not None and fused is None:
             self.residual_position.add(ctx, x)
+        embedded = None
+        if self.keeps_embedding:
+            # the embedding's output as later layers' entries read it: rounded once to the compute dtype
+            embedded = ctx.workspace.get("embedding_out", (ctx.n_tokens, self.width), self.dtype)
+            ops.gather_rows(embedded, x)
         pending = None  # the stream as a SplitStream while a layer has left it split (x is then stale)
         recorded = {}  # this step's lists of launches, by the kind of layer and the state it found the stream in
         for e in self.order:
             block = self.blocks[e.layer]
+            entry = self.entries.get(e.layer)
+            if entry is not None:
+                if pending is not None:
+                    pending.settle()
+                    pending = None
+                entry.forward(x, embedded, ctx)
             cache, state = storage.layer(e.cache_layer), storage.state(e.cache_layer)
             key = None
             if self.replay_layers and phases is None and self._layer_kind[e.layer] is not _OTHER:

@@ -203,3 +203,78 @@ class PostNormGatedBlock:
 
 
 register_block("post_norm_gated", PostNormGatedBlock)
+
+
+class ParallelPairBlock:
+    """x += mixer(c1(norm_mixer(x))) + ffn(c2(norm_ffn(x))): two root-mean-square norms of the same stream (they share the root
+    mean square, so one pass over a row gives both), each followed by a short causal convolution over time of its own, h <- h +
+    conv(h), whose last taps - 1 inputs (the normalised rows, 32-bit) are the layer's per-request state. The convolutions and the
+    feed-forward are optional. Each sublayer adds its result into the 32-bit stream from its last product's epilogue; what they read
+    is a buffer of its own, so both see the stream as the layer found it.
+
+    A slot of the layer's state holds the convolutions' ring first ((taps - 1) places of [sublayers, width] floats, position p at
+    place p % (taps - 1)) and the mixer's own state behind it; the mixer gets its stretch as a `StateSlice`."""
+
+    replayable = True
+    takes_padding_rows = True
+    takes_pending = False
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn, input_conv=None, ffn_conv=None):
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn if ffn is not None else None
+        self.conv, self.ffn_conv = input_conv, ffn_conv if ffn is not None else None
+        self.dtype = mixer.dtype
+        self.mixer_phase = getattr(getattr(spec, "mixer", None), "kind", "mixer")
+        self.ffn_phase = getattr(getattr(spec, "ffn", None), "kind", "ffn")
+        norms = [norm_mixer] + ([norm_ffn] if ffn is not None else [])
+        for norm in norms:
+            if norm is None or not getattr(norm, "root_mean_square", False) or norm.weight is None:
+                raise ValueError("a parallel pair's sublayers each read a weighted root-mean-square norm (kind 'rmsnorm')")
+        if len({float(n.eps) for n in norms}) != 1:
+            raise ValueError("a parallel pair's norms share their root mean square: one epsilon")
+        if ffn is not None and not (hasattr(ffn, "begin") and hasattr(ffn, "finish")):
+            raise ValueError("a parallel pair needs a feed-forward in two halves (begin / finish)")
+        self.eps, self.width = float(norm_mixer.eps), norm_mixer.width
+        self.n_sub = len(norms)
+        self.norm_weights = torch.stack([n.weight for n in norms]).contiguous()
+        convs = [input_conv] + ([self.ffn_conv] if ffn is not None else [])
+        self.taps = max((int(c.taps) for c in convs if c is not None), default=0)
+        self.conv_weights = None
+        if self.taps:
+            if any(c is not None and int(c.taps) != self.taps for c in convs):
+                raise ValueError("a parallel pair's convolutions have one number of taps")
+            zero = torch.zeros((self.width, self.taps), dtype=torch.float32, device=self.norm_weights.device)
+            self.conv_weights = torch.stack([c.weight if c is not None else zero for c in convs]).contiguous()
+        self.ring_floats = max(self.taps - 1, 0) * self.n_sub * self.width
+        own = mixer.state_spec()
+        if own is not None and (len(own.shape) != 1 or own.dtype != "float32"):
+            raise ValueError("a parallel pair keeps its mixer's state behind its own in one flat 32-bit vector a slot")
+        self.mixer_floats = int(own.shape[0]) if own is not None else 0
+
+    def state_spec(self):
+        from ..cache.pages import StateSpec
+
+        total = self.ring_floats + self.mixer_floats
+        return StateSpec((total,)) if total else None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True):
+        ws, n, d, S = ctx.workspace, x.shape[0], x.shape[1], self.n_sub
+        if ctx.phases is not None:
+            ctx.phases.mark(self.mixer_phase)
+        ring = ops.StateSlice(state, 0, self.ring_floats) if self.ring_floats else None
+        h = ws.get("pair_in", (S, n, d), self.dtype)
+        kept = ws.get("pair_normed", (n, S * d), torch.float32) if ring is not None and writes_cache else None
+        ops.norm_shift(h, x, self.norm_weights, 0.0, self.eps, self.conv_weights, ring, ctx, hbuf=kept)
+        # everything that reads the ring has run: the step's last rows take their places in it
+        if kept is not None:
+            ops.ring_keep(ring, self.taps - 1, kept, ctx)
+        begun = self.ffn.begin(h[1], ctx) if self.ffn is not None else None
+        mixer_state = ops.StateSlice(state, self.ring_floats, self.mixer_floats) if self.mixer_floats else None
+        self.mixer.forward(h[0], ctx, cache, mixer_state, x, writes_cache=writes_cache)
+        if self.ffn is not None:
+            if ctx.phases is not None:
+                ctx.phases.mark(self.ffn_phase)
+            self.ffn.finish(begun, ctx, x)
+        return None
+
+
+register_block("parallel_pair", ParallelPairBlock)

@@ -95,3 +95,46 @@ class ClampedGLU:
 
 
 register_ffn("clamped_glu", ClampedGLU)
+
+
+class NormedPowersFFN:
+    """down(c1 N(z) + c2 N(z^2) + c3 N(z^3) + c4) with z = up h, powers entry by entry and N(v) = v / sqrt(mean(v^2) + eps) over the
+    inner width: the first product leaves its 32-bit sums, one kernel takes the three means of a row and mixes the powers, and the inner
+    rows are rounded once, for the second product. The four weights stay on the device."""
+
+    replayable = True
+    takes_padding_rows = True
+
+    def __init__(self, spec, store, dtype: torch.dtype):
+        self.dtype = dtype
+        self.width, self.inner, self.eps = spec.width, spec.inner, float(spec.eps)
+        if int(spec.powers) != 3:
+            raise ValueError(f"a mix of {spec.powers} powers (3 are taken)")
+        t = spec.tensors
+        self.up_weight = store.fetch(t["up"], (self.inner, self.width), "matrix")
+        self.act = store.fetch(t["act"], (4,), "vector")
+        self.down_weight = store.fetch(t["down"], (self.width, self.inner), "matrix")
+
+    def begin(self, h, ctx: StepContext) -> torch.Tensor:
+        """The first product in 32 bits: everything of the feed-forward that reads its input."""
+        z = ctx.workspace.get("powers_in", (h.shape[0], self.inner), torch.float32)
+        linear(h, self.up_weight, None, out=z)
+        return z
+
+    def finish(self, z: torch.Tensor, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        from ..kernels import ops
+
+        inner = ctx.workspace.get("ffn_inner", (z.shape[0], self.inner), self.dtype)
+        ops.normed_powers(inner, z, self.act, self.eps)
+        if out is not None:
+            linear(inner, self.down_weight, None, out=out)
+        else:
+            linear(inner, self.down_weight, None, residual=settled(residual))
+        return None
+
+    def forward(self, h, ctx: StepContext, residual: Optional[torch.Tensor], out: Optional[torch.Tensor] = None):
+        """Adds the result into `residual` (float32 [n, width]), or leaves it in `out`."""
+        return self.finish(self.begin(h, ctx), ctx, residual, out=out)
+
+
+register_ffn("normed_powers_ffn", NormedPowersFFN)

@@ -15,11 +15,13 @@ class LMHead:
     reference's compute_logits after the final norm (src/core/transformer.cpp:2622-2638,
     finish_logits :2613-2620). W may be the token embedding's table (a tied
     head, :1100-1104): the store hands out the same device tensor for the same
-    name, so a tied table is resident once. Logits are float32."""
+    name, so a tied table is resident once. Logits are float32. A spec with a `softcap` bends
+    them last of all: cap * tanh(logits / cap)."""
 
     def __init__(self, spec, store, dtype: torch.dtype):
         self.width, self.vocab_size = spec.width, spec.vocab_size
         self.logit_scale = float(spec.logit_scale)
+        self.softcap = float(getattr(spec, "softcap", 0.0) or 0.0)
         t = spec.tensors
         self.weight = store.fetch(t["weight"], (self.vocab_size, self.width), "table")
         self.bias = store.fetch(t["bias"], (self.vocab_size,), "vector") if "bias" in t else None
@@ -29,6 +31,8 @@ class LMHead:
         linear(h, self.weight, self.bias, out=logits)
         if self.logit_scale != 1.0:
             ops.scale_(logits, self.logit_scale)  # after the bias, as the reference's finish_logits does (:2613-2620)
+        if self.softcap > 0:
+            ops.softcap_(logits, self.softcap)
         return logits
 
 

@@ -28,7 +28,11 @@ class LatentAttention:
     cached rows as keys and as values of one shared head, which is what the paged attention kernels
     do for grouped queries, and the result goes through the head's Wuv. A step reads each cached row
     once for all heads. Scores, softmax and the norm of c are 32-bit; the three projections of h run as
-    one product."""
+    one product.
+
+    Options of the spec: `q_rank` > 0, queries through a latent of their own, q = Wuq (rmsnorm(Wdq h) * w) (the
+    narrow product is left in 32 bits for its norm); `gate_a_head`, a gate of one logit a head (its matrix's
+    rows are repeated over the head's values once, at load, so that the gate stays an epilogue of Wuv's product)."""
 
     replayable = True
     takes_padding_rows = True  # (slot -1: no row of theirs is cached, and no other row attends to them)
@@ -46,11 +50,28 @@ class LatentAttention:
         t = spec.tensors
         H, D, V, R, d = self.n_head, self.head_dim, self.value_dim, self.rank, self.width
         self.q_dim, self.v_dim = H * D, H * V
-        srcs, shapes = [t["q"], t["down"]], [(H * D, d), (R, d)]
-        if self.gated:
-            srcs.append(t["gate"])
-            shapes.append((H * V, d))
-        self.in_weight = store.fetch_joined(srcs, shapes, "matrix", "rows")  # [q | c | gate] of one input
+        self.q_rank = int(getattr(spec, "q_rank", 0) or 0)
+        gate_a_head = bool(getattr(spec, "gate_a_head", False))
+        if self.q_rank or gate_a_head:
+            # [c | gate] of the input; the queries' latent is a product of its own, left in 32 bits for its norm
+            self.q_down = store.fetch(t["q_down"], (self.q_rank, d), "matrix") if self.q_rank else None
+            self.q_down_norm = store.fetch(t["q_down_norm"], (self.q_rank,), "vector") if self.q_rank and "q_down_norm" in t else None
+            self.q_weight = store.fetch(t["q_up"] if self.q_rank else t["q"], (H * D, self.q_rank or d), "matrix")
+            down = store.fetch(t["down"], (R, d), "matrix", keep=False)
+            parts = [down]
+            if self.gated:
+                gate = store.fetch(t["gate"], (H if gate_a_head else H * V, d), "matrix", keep=False)
+                parts.append(gate.repeat_interleave(V, dim=0) if gate_a_head else gate)
+            self.in_weight = store.derived(("latent_in", t["down"].name, t["gate"].name if self.gated else None, V if gate_a_head else 0),
+                                           lambda: torch.cat(parts, dim=0).contiguous())
+            self.q_dim = 0  # (no queries among the joint product's columns)
+        else:
+            self.q_weight = None
+            srcs, shapes = [t["q"], t["down"]], [(H * D, d), (R, d)]
+            if self.gated:
+                srcs.append(t["gate"])
+                shapes.append((H * V, d))
+            self.in_weight = store.fetch_joined(srcs, shapes, "matrix", "rows")  # [q | c | gate] of one input
         self.down_norm = store.fetch(t["down_norm"], (R,), "vector") if "down_norm" in t else None
         up_k = store.fetch(t["up_k"], (H * D, R), "matrix")
         # a head's Wuk^T, [rank, head_dim] with the head's dimensions contiguous: what multiplies its query
@@ -79,7 +100,18 @@ class LatentAttention:
         if writes_cache:
             ops.latent_store(rows, proj, self.q_dim, self.down_norm, self.eps, group.slots)
         q_c = ws.get("latent_q", (n, H * R), self.dtype)
-        ops.heads_product(q_c, proj[:, :self.q_dim], self.up_k_t)
+        if self.q_weight is not None:
+            q_in = h
+            if self.q_rank:
+                low = ws.get("latent_q_low", (n, self.q_rank), torch.float32)
+                linear(h, self.q_down, None, out=low)
+                q_in = ws.get("latent_q_normed", (n, self.q_rank), self.dtype)
+                ops.rmsnorm(q_in, low, self.q_down_norm, self.eps)
+            queries = ws.get("latent_queries", (n, H * self.head_dim), self.dtype)
+            linear(q_in, self.q_weight, None, out=queries)
+        else:
+            queries = proj[:, :self.q_dim]
+        ops.heads_product(q_c, queries, self.up_k_t)
         att = ws.get("latent_att", (n, H * R), self.dtype)
         splits = ops.attention(att, q_c, rows, rows, group.block_tables, ctx, n_head=H, scale=self.scale, window=self.window)
         assert splits is None

@@ -88,7 +88,8 @@ class RMSNorm:
     """y = x / sqrt(mean(x^2) + eps) * weight over the last axis, the epsilon inside the root; sums and
     scaling 32-bit. `rows` gathers (the final norm runs on the wanted rows only). Behind a sublayer,
     a block applies it through the fused residual update (`ops.gated_norm_add`), which reads
-    `weight` and `eps` from here."""
+    `weight` and `eps` from here. A spec with a `weight_offset` stores its weight around zero: what
+    multiplies is weight + offset, added once at load in 32 bits."""
 
     replayable = True
     takes_padding_rows = True
@@ -100,6 +101,10 @@ class RMSNorm:
         self.dtype = dtype
         w = spec.tensors.get("weight")
         self.weight = store.fetch(w, (self.width,), "vector") if w is not None else None
+        offset = float(getattr(spec, "weight_offset", 0.0) or 0.0)
+        if offset and self.weight is not None:
+            stored = self.weight
+            self.weight = store.derived(("weight_plus", w.name, offset), lambda: (stored + offset).contiguous())
 
     def forward(self, x: torch.Tensor, ctx: StepContext, rows: Optional[torch.Tensor] = None,
                 n_rows: Optional[int] = None, name: str = "normed") -> torch.Tensor:

@@ -14,7 +14,7 @@ from ..errors import Unsupported
 
 _REGISTRIES: Dict[str, Dict[str, type]] = {
     "mixer": {}, "ffn": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
-    "conv": {}, "gate": {},
+    "conv": {}, "gate": {}, "entry": {},
 }
 
 
@@ -32,6 +32,7 @@ def register_embedding(kind: str, cls: type) -> type: return _register("embeddin
 def register_head(kind: str, cls: type) -> type: return _register("head", kind, cls)
 def register_conv(kind: str, cls: type) -> type: return _register("conv", kind, cls)
 def register_gate(kind: str, cls: type) -> type: return _register("gate", kind, cls)
+def register_entry(kind: str, cls: type) -> type: return _register("entry", kind, cls)
 
 
 def find_part(family: str, kind: str) -> type:
