@@ -6,7 +6,7 @@
     python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
     python bench.py --link-floor                     # what one dependent kernel of a replayed graph costs at least
     python bench.py --product 4096,4096,16384,8,15   # one product in tiles of 128 x 128 and of 256 x 256
-    python bench.py --design bokulix|mofulix [--design-sizes small,medium,xl] [--layers L] [--phases]   # that design beside GPT-2 at equal sizes
+    python bench.py --design bokulix|mofulix|dopilorn [--design-sizes small,medium,xl] [--layers L] [--phases]   # that design beside GPT-2 (dopilorn: beside Mofulix) at equal sizes
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -483,8 +483,92 @@ def mofulix_prefill_flops(cfg, prompt_lens, logit_rows):
     return flops
 
 
+
+# -- Dopilorn beside Mofulix at equal sizes -------------------------------------------------------------------
+# The Dopilorn of each size has GPT-2's width, layers, vocabulary and head count; its layers take turns as a delta-rule recurrence
+# (heads of 64, a decay of rank 64), attention in two maps a head (maps of 32, values of 64, as many key heads as query heads, a
+# convolution of four taps on the projections, a window as long as the context, so that each map walks every key) and latent
+# attention (heads of 64 over cached rows of 128, 256 at XL's width, queries through a latent of half the width); two norms and
+# two convolutions of four taps a layer; a feed-forward of two matrices as wide as GPT-2's. It stands beside Mofulix, the engine's
+# other design of parallel layers that mixes recurrences with attention.
+def dopilorn_config(gpt2_cfg):
+    d, H, F, L = gpt2_cfg["n_embd"], gpt2_cfg["n_head"], gpt2_cfg["n_inner"], gpt2_cfg["n_layer"]
+    hd = d // H
+    mlp = {"kind": "dense", "ff": F}
+    kinds = [
+        {"type": "general_delta", "mixer": {"heads": H, "dim": hd, "decay_rank": 64}},
+        {"type": "attention", "mixer": {"heads": H, "kv_heads": H, "dim": hd // 2, "vdim": hd, "scale": (hd // 2) ** -0.5, "diff": 0.5, "conv": 4,
+                                        "mask": {"size": gpt2_cfg["n_positions"]}}},
+        {"type": "latent_attention", "mixer": {"heads": H, "dim": hd, "vdim": hd, "kv_rank": 256 if d >= 1600 else 128, "q_rank": d // 2 // 64 * 64,
+                                               "scale": hd ** -0.5}},
+    ]
+    layers = [dict(json.loads(json.dumps(kinds[i % 3])), mlp=dict(mlp)) for i in range(L)]
+    return {"architecture": "Dopilorn", "vocab": gpt2_cfg["vocab_size"], "width": d, "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "logit_softcap": 30.0,
+            "max_positions": gpt2_cfg["n_positions"], "layers": layers}
+
+
+def _dopilorn_layer_weights(entry, d):
+    """Matrix elements of a layer (what a step reads of it; all of them are products' operands, 2 flops an element a token)."""
+    m, kind = entry["mixer"], entry["type"]
+    n = 2 * entry["mlp"]["ff"] * d if entry.get("mlp") else 0
+    H, D = m["heads"], m["dim"]
+    if kind == "general_delta":
+        R = m.get("decay_rank", 16)
+        n += 5 * H * D * d + R * d + H * D * R + d * H * D
+    elif kind == "attention":
+        G, V = m.get("kv_heads", H), m.get("vdim", D)
+        n += (2 * H * D + 2 * G * D + G * V) * d + d * H * V
+    else:
+        V, R, Q = m["vdim"], m["kv_rank"], m["q_rank"]
+        n += (Q + R + H) * d + H * D * Q + H * (D + V) * R + d * H * V
+    return n
+
+
+def dopilorn_step_bytes(cfg, batch):
+    """The bytes a decode step has to read: every matrix once, the head, the cached rows inside the windows (two planes of keys
+    and one of values, padded to one width; one latent row), and the 32-bit state of the recurrent layers (read and written)."""
+    def step_bytes(contexts, steps, elt):
+        d, V = cfg["width"], cfg["vocab"]
+        total = V * d * elt
+        for entry in cfg["layers"]:
+            m = entry["mixer"]
+            total += _dopilorn_layer_weights(entry, d) * elt
+            if entry["type"] == "general_delta":
+                total += len(contexts) * 2 * m["heads"] * m["dim"] * m["dim"] * 4
+            elif entry["type"] == "attention":
+                window = (m.get("mask") or {}).get("size", 0)
+                seen = sum(sum(min(c + s + 1, window) if window else c + s + 1 for s in range(steps)) for c in contexts) / max(steps, 1)
+                P = -(-max(m["dim"], m.get("vdim", m["dim"])) // 8) * 8
+                total += seen * 3 * m.get("kv_heads", m["heads"]) * P * elt
+            else:
+                seen = sum(sum(c + s + 1 for s in range(steps)) for c in contexts) / max(steps, 1)
+                total += seen * m["kv_rank"] * elt
+        return total
+    return step_bytes
+
+
+def dopilorn_prefill_flops(cfg, prompt_lens, logit_rows):
+    d, V, n = cfg["width"], cfg["vocab"], sum(prompt_lens)
+    flops = 2.0 * logit_rows * d * V
+    for entry in cfg["layers"]:
+        m = entry["mixer"]
+        flops += 2.0 * n * _dopilorn_layer_weights(entry, d)
+        if entry["type"] == "general_delta":
+            flops += n * m["heads"] * 8.0 * m["dim"] * m["dim"]  # a token: what the key sees, the state's update, its read, a head
+        elif entry["type"] == "attention":
+            window = (m.get("mask") or {}).get("size", 0)
+            pairs = sum(sum(min(i + 1, window) if window else i + 1 for i in range(t)) for t in prompt_lens)
+            flops += 2.0 * pairs * m["heads"] * 2 * (m["dim"] + m.get("vdim", m["dim"]))
+        else:
+            pairs = sum(t * (t + 1) / 2 for t in prompt_lens)
+            flops += 2.0 * pairs * m["heads"] * 2 * m["kv_rank"]
+    return flops
+
+
 DESIGNS = {"bokulix": (lambda gpt2, size: bokulix_config(gpt2, BOKULIX_SHAPES[size]), bokulix_step_bytes, bokulix_prefill_flops),
-           "mofulix": (lambda gpt2, size: mofulix_config(gpt2), mofulix_step_bytes, mofulix_prefill_flops)}
+           "mofulix": (lambda gpt2, size: mofulix_config(gpt2), mofulix_step_bytes, mofulix_prefill_flops),
+           "dopilorn": (lambda gpt2, size: dopilorn_config(gpt2), dopilorn_step_bytes, dopilorn_prefill_flops)}
+BESIDE = {"dopilorn": "mofulix"}  # the engine's closest model, where that is not GPT-2
 
 
 def design_run(args):
@@ -499,9 +583,10 @@ def design_run(args):
         gpt2 = dict(SMALL, **SIZES[size])
         if args.layers:
             gpt2["n_layer"] = args.layers
-        designs = {"gpt2": gpt2, args.design: make_config(gpt2, size)}
+        beside = BESIDE.get(args.design, "gpt2")
+        designs = {beside: gpt2 if beside == "gpt2" else DESIGNS[beside][0](gpt2, size), args.design: make_config(gpt2, size)}
         if args.design_only:
-            del designs["gpt2"]
+            del designs[beside]
         ctx = gpt2["n_positions"]
         k = max(16, min(args.steps, 128, ctx - args.prompt - 16))
         for name, cfg in designs.items():
@@ -510,14 +595,14 @@ def design_run(args):
                 engine = make_engine(d, args.dtype, 64, ctx, page_size=args.page_size, phases=args.phases)
                 lens = [1024, 1024]
                 ptps, pms = prefill_run(engine, cfg, lens)
-                flops = flops_of(cfg, lens, 2) if name != "gpt2" else prefill_flops(cfg, lens, 2)
+                flops = DESIGNS[name][2](cfg, lens, 2) if name != "gpt2" else prefill_flops(cfg, lens, 2)
                 run = {"design": name, "size": size, "layers": gpt2["n_layer"],
                        "prefill": {"tokens": 2048, "tok_s": round(ptps, 1), "ms": round(pms, 4), "gflop": round(flops / 1e9, 1),
                                    "frac_of_matrix_peak": round(flops / (pms * 1e-3) / MFMA_PEAK[short], 4)}}
                 if args.phases:
                     run["prefill"]["phases_ms"] = {n: round(v / 7, 4) for n, v in engine.phases_ms(reset=True).items()}  # (prefill_run steps 7 times)
                 for b in (1, 8, 64):
-                    bytes_fn = step_bytes_of(cfg, b) if name != "gpt2" else None
+                    bytes_fn = DESIGNS[name][1](cfg, b) if name != "gpt2" else None
                     t, ms, nbytes = decode_run(engine, cfg, b, args.prompt, k, 4, step_bytes=bytes_fn)
                     run[f"decode_b{b}"] = {"tok_s": round(t, 1), "ms_per_step": round(ms, 4), "mbytes_per_step": round(nbytes / 1e6, 1),
                                            "frac_of_hbm_peak": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
@@ -529,7 +614,7 @@ def design_run(args):
                         run[f"decode_b{b}"]["phases_ms"] = {n: round(max(v - prompts.get(n, 0.0), 0.0) / (k + 4), 4) for n, v in whole.items()}
                 runs.append(run)
                 del engine
-    print(json.dumps({"metric": f"{args.design.capitalize()} beside GPT-2 at equal layer sizes: prefill of 2,048 tokens and decode steps", "dtype": short,
+    print(json.dumps({"metric": f"{args.design.capitalize()} beside {BESIDE.get(args.design, 'GPT-2').capitalize() if args.design in BESIDE else 'GPT-2'} at equal layer sizes: prefill of 2,048 tokens and decode steps", "dtype": short,
                       "data": "synthetic", "page_size": args.page_size, "prompt_len": args.prompt, "runs": runs}))
     return 0
 
@@ -561,8 +646,9 @@ def main():
     ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
     ap.add_argument("--phases", action="store_true", help="device milliseconds per phase of the forward pass (embed, attention, dense_ffn, lm_head) a decode step "
                     "and a prefill of 2,048 tokens, as the reference's command line prints them (tools/liyab_cli.cpp:198-211); steps run kernel by kernel, without graphs")
-    ap.add_argument("--design", default="", choices=["", "bokulix", "mofulix"],
-                    help="bokulix, mofulix: that design beside GPT-2 at equal layer sizes (prefill and decode, both with their rooflines)")
+    ap.add_argument("--design", default="", choices=["", "bokulix", "mofulix", "dopilorn"],
+                    help="bokulix, mofulix: that design beside GPT-2 at equal layer sizes (prefill and decode, both with their rooflines); "
+                         "dopilorn: beside Mofulix, the engine's closest model")
     ap.add_argument("--design-only", action="store_true", help="with --design: skip the GPT-2 run (for profiling)")
     ap.add_argument("--design-sizes", default="small,medium,xl", help="the sizes --design runs (of small, medium, xl)")
     args = ap.parse_args()

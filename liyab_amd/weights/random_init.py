@@ -62,7 +62,7 @@ class DrawingStore:
     def has(self, src: TensorSource) -> bool:
         return src.required or src.name in self.tensors
 
-    def fetch(self, src: TensorSource, shape: Sequence[int], role: str) -> Optional[torch.Tensor]:
+    def fetch(self, src: TensorSource, shape: Sequence[int], role: str, keep: bool = True) -> Optional[torch.Tensor]:
         if not src.required and src.name not in self.tensors:
             return None  # an optional tensor stays absent
         shape = tuple(int(s) for s in shape)

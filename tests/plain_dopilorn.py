@@ -157,12 +157,12 @@ def run_order(cfg):
 def layer(x, t, i, entry, cfg):
     eps = cfg["norm"]["eps"]
     p = f"l{i}."
-    unit_x = unit(x, eps)
-    hm, hf = unit_x * (1.0 + t[p + "norm1"]), unit_x * (1.0 + t[p + "norm2"])
+    hm = offset_norm(x, t[p + "norm1"], eps)
     if cfg.get("canon"):
         hm = hm + time_conv(hm, t[p + "canon1"])
     y = MIXERS[entry["type"]](hm, t, p + "mix.", entry["mixer"], eps)
     if entry.get("mlp") is not None:
+        hf = offset_norm(x, t[p + "norm2"], eps)
         if cfg.get("canon"):
             hf = hf + time_conv(hf, t[p + "canon2"])
         y = y + feed_forward(hf, t, p + "mlp.", eps)
