@@ -17,6 +17,7 @@
 namespace liyab {
 
 constexpr int kMapsMaxTaps = 16;
+constexpr int kMapsUnits = 8;  // units a workgroup: two a wave
 
 struct MapsArgs {
     const float* src;   // [n, ld]
@@ -57,38 +58,143 @@ maps_store_kernel(MapsArgs a) {
     const int cache_slot = a.slots[t];
     const bool cached = cache_slot >= 0 && cache_slot < a.num_pages * a.page_size;
     const int page = cached ? cache_slot / a.page_size : 0, off = cached ? cache_slot % a.page_size : 0;
-    const int nq = 2 * H * P, nk = 2 * G * P, nv = G * P;
-    for (int e = threadIdx.x; e < nq + nk + nv; e += 256) {
-        int c = -1;  // the projection's channel this element holds, or none (padding)
+    const int nq = 2 * H * P;
+    // a unit: one head's P entries of one destination (queries of a map, keys of a map, values); a wave a unit, kMapsUnits a
+    // workgroup, so that a step of few rows still spreads over the chip
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
+    const int n_units = 2 * H + 3 * G;
+    const int unit_end = min(n_units, static_cast<int>(blockIdx.y + 1) * kMapsUnits);
+    for (int unit = blockIdx.y * kMapsUnits + wave; unit < unit_end; unit += 256 / kWave) {
+        int c0, width;  // the projection's first channel of this unit and how many it has (the rest of P is padding)
         T* dst = nullptr;
-        if (e < nq) {
-            const int m = e / (H * P), h = (e / P) % H, i = e % P;
-            if (i < D) c = h * 2 * D + m * D + i;
-            dst = static_cast<T*>(a.q_out) + static_cast<int64_t>(t) * nq + e;
-        } else if (e < nq + nk) {
-            const int f = e - nq;
-            const int m = f / (G * P), g = (f / P) % G, i = f % P;
-            if (i < D) c = 2 * H * D + g * 2 * D + m * D + i;
-            if (cached) dst = static_cast<T*>(m == 0 ? a.k1 : a.k2) + ((static_cast<int64_t>(page) * G + g) * a.page_size + off) * P + i;
+        if (unit < 2 * H) {
+            const int m = unit / H, h = unit % H;
+            c0 = h * 2 * D + m * D;
+            width = D;
+            dst = static_cast<T*>(a.q_out) + static_cast<int64_t>(t) * nq + static_cast<int64_t>(unit) * P;
+        } else if (unit < 2 * H + 2 * G) {
+            const int f = unit - 2 * H;
+            const int m = f / G, g = f % G;
+            c0 = 2 * H * D + g * 2 * D + m * D;
+            width = D;
+            if (cached) dst = static_cast<T*>(m == 0 ? a.k1 : a.k2) + ((static_cast<int64_t>(page) * G + g) * a.page_size + off) * P;
         } else {
-            const int f = e - nq - nk;
-            const int g = f / P, i = f % P;
-            if (i < V) c = 2 * H * D + 2 * G * D + g * V + i;
-            if (cached) dst = static_cast<T*>(a.vc) + ((static_cast<int64_t>(page) * G + g) * a.page_size + off) * P + i;
+            const int g = unit - 2 * H - 2 * G;
+            c0 = 2 * H * D + 2 * G * D + g * V;
+            width = V;
+            if (cached) dst = static_cast<T*>(a.vc) + ((static_cast<int64_t>(page) * G + g) * a.page_size + off) * P;
         }
         if (dst == nullptr) continue;
-        float acc = 0.0f;
-        if (c >= 0) {
-            if (a.cw == nullptr) acc = row[c];
-            else {
-                const float* w = a.cw + static_cast<int64_t>(c) * a.taps;
-                acc = w[a.taps - 1] * row[c];
+        for (int i = lane; i < P; i += kWave) {
+            float acc = 0.0f;
+            if (i < width) {
+                const int c = c0 + i;
+                if (a.cw == nullptr) acc = row[c];
+                else {
+                    const float* w = a.cw + static_cast<int64_t>(c) * a.taps;
+                    acc = w[a.taps - 1] * row[c];
 #pragma unroll
-                for (int m = 1; m < kMapsMaxTaps; ++m)
-                    if (m <= ring && src[m] != nullptr) acc += w[a.taps - 1 - m] * src[m][c];
+                    for (int m = 1; m < kMapsMaxTaps; ++m)
+                        if (m <= ring && src[m] != nullptr) acc += w[a.taps - 1 - m] * src[m][c];
+                }
             }
+            dst[i] = from_float<T>(acc);
         }
-        *dst = from_float<T>(acc);
+    }
+}
+
+// The same for head sizes that are multiples of four (and rows that start at multiples of 16 bytes): a thread takes four channels
+// side by side of one row, a workgroup 1,024 of a row's channels, so that every load is 16 bytes wide and all of a thread's
+// loads are on their way together; the zeros behind the narrower heads are written after that.
+template <typename T>
+__device__ __forceinline__ void store4(T* dst, const float (&v)[4]);
+template <>
+__device__ __forceinline__ void store4<float>(float* dst, const float (&v)[4]) {
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
+    *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float (&v)[4]) {
+    typedef __attribute__((ext_vector_type(4))) unsigned short u16x4;
+    *reinterpret_cast<u16x4*>(dst) = u16x4{from_float<bf16_t>(v[0]), from_float<bf16_t>(v[1]), from_float<bf16_t>(v[2]), from_float<bf16_t>(v[3])};
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+maps_store_vec_kernel(MapsArgs a) {
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
+    const int t = blockIdx.x;
+    const int s = a.tok_seq[t], p = a.positions[t];
+    const int in_step = t - a.seq_starts[s];
+    const int ring = a.taps > 0 ? a.taps - 1 : 0;
+    int slot = a.state_slots[s];
+    if (slot < 0 || slot >= a.n_slots || a.state == nullptr) slot = -1;
+    const int H = a.H, G = a.G, D = a.D, V = a.V, P = a.P;
+    const int QC = 2 * H * D, KC = 2 * G * D, C = QC + KC + G * V;
+    const float* src[kMapsMaxTaps];  // the row m back, or null
+#pragma unroll
+    for (int m = 1; m < kMapsMaxTaps; ++m) {
+        src[m] = nullptr;
+        if (m <= ring && p - m >= 0) {
+            if (m <= in_step) src[m] = a.src + static_cast<int64_t>(t - m) * a.ld;
+            else if (slot >= 0) src[m] = a.state + static_cast<int64_t>(slot) * a.state_stride + static_cast<int64_t>((p - m) % ring) * C;
+        }
+    }
+    const float* row = a.src + static_cast<int64_t>(t) * a.ld;
+    const int cache_slot = a.slots[t];
+    const bool cached = cache_slot >= 0 && cache_slot < a.num_pages * a.page_size;
+    const int page = cached ? cache_slot / a.page_size : 0, off = cached ? cache_slot % a.page_size : 0;
+    const int64_t nq = 2LL * H * P;
+    T* const q_row = static_cast<T*>(a.q_out) + static_cast<int64_t>(t) * nq;
+    auto paged = [&](void* plane, int g) { return static_cast<T*>(plane) + ((static_cast<int64_t>(page) * G + g) * a.page_size + off) * P; };
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (c < C) {
+        T* dst = nullptr;
+        if (c < QC) {
+            const int h = c / (2 * D), r = c % (2 * D);
+            dst = q_row + static_cast<int64_t>((r / D) * H + h) * P + r % D;
+        } else if (c < QC + KC) {
+            const int f = c - QC;
+            const int g = f / (2 * D), r = f % (2 * D);
+            if (cached) dst = paged(r / D == 0 ? a.k1 : a.k2, g) + r % D;
+        } else {
+            const int f = c - QC - KC;
+            if (cached) dst = paged(a.vc, f / V) + f % V;
+        }
+        if (dst != nullptr) {
+            const f32x4 x0 = *reinterpret_cast<const f32x4*>(row + c);
+            float acc[4] = {x0[0], x0[1], x0[2], x0[3]};
+            if (a.cw != nullptr) {
+                const float* w = a.cw + static_cast<int64_t>(c) * a.taps + a.taps - 1;  // (the newest tap of the first channel)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] *= w[e * a.taps];
+#pragma unroll
+                for (int m = 1; m < kMapsMaxTaps; ++m) {
+                    if (m <= ring && src[m] != nullptr) {
+                        const f32x4 xm = *reinterpret_cast<const f32x4*>(src[m] + c);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[e] += w[e * a.taps - m] * xm[e];
+                    }
+                }
+            }
+            store4<T>(dst, acc);
+        }
+    }
+    // zeros behind the heads' own entries
+    const int pad_k = P - D, pad_v = P - V;
+    const int n_qpad = 2 * H * pad_k, n_kpad = 2 * G * pad_k, n_vpad = G * pad_v;
+    for (int e = blockIdx.y * 256 + threadIdx.x; e < n_qpad + n_kpad + n_vpad; e += gridDim.y * 256) {
+        T* dst = nullptr;
+        if (e < n_qpad) dst = q_row + static_cast<int64_t>(e / pad_k) * P + D + e % pad_k;
+        else if (e < n_qpad + n_kpad) {
+            const int f = e - n_qpad;
+            const int unit = f / pad_k;
+            if (cached) dst = paged(unit / G == 0 ? a.k1 : a.k2, unit % G) + D + f % pad_k;
+        } else {
+            const int f = e - n_qpad - n_kpad;
+            if (cached) dst = paged(a.vc, f / pad_v) + V + f % pad_v;
+        }
+        if (dst != nullptr) *dst = from_float<T>(0.0f);
     }
 }
 
@@ -131,8 +237,17 @@ extern "C" int liyab_maps_store(const float* src, int64_t ld, const float* cw, i
     if (n == 0) return 0;
     MapsArgs a{src, ld, cw, taps, state, state_stride, n_slots, q_out, k1, k2, vc, slots, page_size, num_pages, tok_seq, positions, seq_starts,
                state_slots, H, G, D, V, P};
-    if (dtype == kF32) maps_store_kernel<float><<<n, 256, 0, stream>>>(a);
-    else maps_store_kernel<bf16_t><<<n, 256, 0, stream>>>(a);
+    const auto at16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+    if (D % 4 == 0 && V % 4 == 0 && ld % 4 == 0 && at16(src) && at16(q_out) && at16(k1) && at16(k2) && at16(vc) &&
+        (state == nullptr || (at16(state) && state_stride % 4 == 0))) {
+        const dim3 grid(n, static_cast<unsigned>((C / 4 + 255) / 256));
+        if (dtype == kF32) maps_store_vec_kernel<float><<<grid, 256, 0, stream>>>(a);
+        else maps_store_vec_kernel<bf16_t><<<grid, 256, 0, stream>>>(a);
+        return check_launch("maps_store");
+    }
+    const dim3 grid(n, (2 * H + 3 * G + kMapsUnits - 1) / kMapsUnits);
+    if (dtype == kF32) maps_store_kernel<float><<<grid, 256, 0, stream>>>(a);
+    else maps_store_kernel<bf16_t><<<grid, 256, 0, stream>>>(a);
     return check_launch("maps_store");
 }
 

@@ -1704,6 +1704,25 @@ def delta_takes(head_dim: int) -> bool:
     return 1 <= head_dim <= 256
 
 
+def delta_segments_from(n: int, n_seqs: int) -> bool:
+    """Whether a step of n rows of n_seqs requests walks its delta-rule recurrences in segments side by side: when some request
+    may bring SCAN_SEGMENT_FROM rows or more. It follows from the step's rows and requests alone (as the grids do), so that a
+    captured graph of such a step holds for every step of its shape; a step of short portions only that walks in segments
+    all the same computes the same recurrence in three launches."""
+    return n - n_seqs + 1 >= SCAN_SEGMENT_FROM
+
+
+def _delta_segments(ctx, n: int, n_head: int, head_dim: int):
+    """(tokens a segment, the most segments, scratch for the segments' ends, transitions and starts), or (0, 0, None, None, None)."""
+    if not delta_segments_from(n, ctx.n_seqs):
+        return 0, 0, None, None, None
+    most = -(-n // SCAN_SEGMENT) + ctx.n_seqs
+    state = ctx.workspace.get("delta_seg_state", (most, n_head, head_dim, head_dim), torch.float32)
+    trans = ctx.workspace.get("delta_seg_trans", (most, n_head, head_dim, head_dim), torch.float32)
+    start = ctx.workspace.get("delta_seg_start", (most, n_head, head_dim, head_dim), torch.float32)
+    return SCAN_SEGMENT, most, state.data_ptr(), trans.data_ptr(), start.data_ptr()
+
+
 def delta_rule(out: torch.Tensor, proj: torch.Tensor, wraw: torch.Tensor, w0: torch.Tensor, a_bias: torch.Tensor, norm_w: Optional[torch.Tensor],
                eps: float, state: StateSlice, ctx, *, n_head: int, head_dim: int, decay_scale: float, key_eps: float) -> None:
     """The decayed delta rule over each request's rows of the step. proj float32 [n, >= 5 * H * D] = [r | k | v | removal logits |
@@ -1730,7 +1749,8 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, wraw: torch.Tensor, w0: to
     _lib.call("liyab_delta_prepare", prep.data_ptr(), p + 4 * HD, wraw.data_ptr(), p + 12 * HD, ld, ldw, w0.data_ptr(), a_bias.data_ptr(),
               float(decay_scale), float(key_eps), n, H, D, _stream())
     _lib.call("liyab_delta_scan", o.data_ptr(), p, p + 4 * HD, p + 8 * HD, ld, prep.data_ptr(), state.data_ptr(), state.stride, state.n_slots,
-              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, H, D, _stream())
+              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, H, D, *_delta_segments(ctx, n, H, D),
+              _stream())
     _lib.call("liyab_head_norm_gate", out.data_ptr(), dtype_code(out.dtype), o.data_ptr(), p + 16 * HD, ld, _ptr(norm_w), float(eps), n, H, D, _stream())
 
 
