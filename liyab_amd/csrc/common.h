@@ -42,6 +42,20 @@ __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
 
+// Four values side by side to dst (aligned to four of its elements), rounded as from_float rounds one.
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+template <typename T>
+__device__ __forceinline__ void store4(T* dst, const float (&v)[4]);
+template <>
+__device__ __forceinline__ void store4<float>(float* dst, const float (&v)[4]) {
+    *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{v[0], v[1], v[2], v[3]};
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float (&v)[4]) {
+    typedef __attribute__((ext_vector_type(4))) unsigned short u16x4;
+    *reinterpret_cast<u16x4*>(dst) = u16x4{float_to_bf16(v[0]), float_to_bf16(v[1]), float_to_bf16(v[2]), float_to_bf16(v[3])};
+}
+
 // Stores `code`'s message for liyab_last_error(); returns `code`.
 int fail(int code, const char* fmt, ...);
 // 0, or fail(...) with the runtime's message when the last launch failed.

@@ -3,7 +3,7 @@
 //
 // liyab_maps_store: from a projection's 32-bit rows [q | k | v] (a query head holds [map 1 | map 2], D values each; a key head
 //   the same; a value head V values), every channel first through a causal convolution over time when there is one,
-//       y_t = sum_{j < taps} c[:, j] * u_(t - taps + 1 + j)          (zeros before a request's start)
+//       y_t = sum_{j < taps} c[j, :] * u_(t - taps + 1 + j)          (zeros before a request's start; c is [taps, C])
 //   whose earlier inputs come from the step's own rows or from the request's history (position p at ring place p % (taps - 1) of
 //   its slot, [C] floats a place, kept by liyab_ring_keep after this kernel has run), to
 //     queries  [n, 2, H, P]  (map-major, so that each map is a set of H heads of P for the attention kernels),
@@ -22,7 +22,7 @@ constexpr int kMapsUnits = 8;  // units a workgroup: two a wave
 struct MapsArgs {
     const float* src;   // [n, ld]
     int64_t ld;
-    const float* cw;    // [C, taps] or null
+    const float* cw;    // [taps, C] or null
     int taps;
     const float* state; // the ring of slot 0; a slot is state_stride floats further
     int64_t state_stride;
@@ -91,11 +91,11 @@ maps_store_kernel(MapsArgs a) {
                 const int c = c0 + i;
                 if (a.cw == nullptr) acc = row[c];
                 else {
-                    const float* w = a.cw + static_cast<int64_t>(c) * a.taps;
-                    acc = w[a.taps - 1] * row[c];
+                    const float* w = a.cw + static_cast<int64_t>(a.taps - 1) * C + c;  // (the newest tap; a tap's channels lie side by side)
+                    acc = w[0] * row[c];
 #pragma unroll
                     for (int m = 1; m < kMapsMaxTaps; ++m)
-                        if (m <= ring && src[m] != nullptr) acc += w[a.taps - 1 - m] * src[m][c];
+                        if (m <= ring && src[m] != nullptr) acc += w[-static_cast<int64_t>(m) * C] * src[m][c];
                 }
             }
             dst[i] = from_float<T>(acc);
@@ -106,19 +106,6 @@ maps_store_kernel(MapsArgs a) {
 // The same for head sizes that are multiples of four (and rows that start at multiples of 16 bytes): a thread takes four channels
 // side by side of one row, a workgroup 1,024 of a row's channels, so that every load is 16 bytes wide and all of a thread's
 // loads are on their way together; the zeros behind the narrower heads are written after that.
-template <typename T>
-__device__ __forceinline__ void store4(T* dst, const float (&v)[4]);
-template <>
-__device__ __forceinline__ void store4<float>(float* dst, const float (&v)[4]) {
-    typedef __attribute__((ext_vector_type(4))) float f32x4;
-    *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-}
-template <>
-__device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float (&v)[4]) {
-    typedef __attribute__((ext_vector_type(4))) unsigned short u16x4;
-    *reinterpret_cast<u16x4*>(dst) = u16x4{from_float<bf16_t>(v[0]), from_float<bf16_t>(v[1]), from_float<bf16_t>(v[2]), from_float<bf16_t>(v[3])};
-}
-
 template <typename T>
 __global__ void __launch_bounds__(256)
 maps_store_vec_kernel(MapsArgs a) {
@@ -165,15 +152,16 @@ maps_store_vec_kernel(MapsArgs a) {
             const f32x4 x0 = *reinterpret_cast<const f32x4*>(row + c);
             float acc[4] = {x0[0], x0[1], x0[2], x0[3]};
             if (a.cw != nullptr) {
-                const float* w = a.cw + static_cast<int64_t>(c) * a.taps + a.taps - 1;  // (the newest tap of the first channel)
+                const float* w = a.cw + static_cast<int64_t>(a.taps - 1) * C + c;  // (the newest tap of four channels side by side)
+                const f32x4 w0 = *reinterpret_cast<const f32x4*>(w);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) acc[e] *= w[e * a.taps];
+                for (int e = 0; e < 4; ++e) acc[e] *= w0[e];
 #pragma unroll
                 for (int m = 1; m < kMapsMaxTaps; ++m) {
                     if (m <= ring && src[m] != nullptr) {
-                        const f32x4 xm = *reinterpret_cast<const f32x4*>(src[m] + c);
+                        const f32x4 xm = *reinterpret_cast<const f32x4*>(src[m] + c), wm = *reinterpret_cast<const f32x4*>(w - static_cast<int64_t>(m) * C);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[e] += w[e * a.taps - m] * xm[e];
+                        for (int e = 0; e < 4; ++e) acc[e] += wm[e] * xm[e];
                     }
                 }
             }
@@ -238,7 +226,7 @@ extern "C" int liyab_maps_store(const float* src, int64_t ld, const float* cw, i
     MapsArgs a{src, ld, cw, taps, state, state_stride, n_slots, q_out, k1, k2, vc, slots, page_size, num_pages, tok_seq, positions, seq_starts,
                state_slots, H, G, D, V, P};
     const auto at16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-    if (D % 4 == 0 && V % 4 == 0 && ld % 4 == 0 && at16(src) && at16(q_out) && at16(k1) && at16(k2) && at16(vc) &&
+    if (D % 4 == 0 && V % 4 == 0 && ld % 4 == 0 && at16(src) && at16(cw) && at16(q_out) && at16(k1) && at16(k2) && at16(vc) &&
         (state == nullptr || (at16(state) && state_stride % 4 == 0))) {
         const dim3 grid(n, static_cast<unsigned>((C / 4 + 255) / 256));
         if (dtype == kF32) maps_store_vec_kernel<float><<<grid, 256, 0, stream>>>(a);

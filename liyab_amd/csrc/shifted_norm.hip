@@ -2,7 +2,8 @@
 //
 // liyab_norm_shift: one pass over a row of the 32-bit stream gives every sublayer its input:
 //   h_s = x / sqrt(mean(x^2) + eps) * (w_s + offset),            s = 0 .. S - 1 (the sublayers share the root mean square)
-//   out_s[t] = h_s[t] + sum_{j < taps} c_s[:, j] * h_s[t - taps + 1 + j]     (zeros before a request's start; no c: out = h)
+//   out_s[t] = h_s[t] + sum_{j < taps} c_s[j, :] * h_s[t - taps + 1 + j]     (zeros before a request's start; no c: out = h;
+//                                                                              c is [S, taps, d]: a tap's channels side by side)
 // A source row inside the step's portion is normalised again by the workgroup that needs it (the same arithmetic in the
 // same order as its own workgroup's, so the same bits); an earlier one is read, already normalised, from the request's
 // history: position p at ring place p % (taps - 1) of state[slot], each place holding [S, d] floats. `hbuf` [n, S * d]
@@ -88,16 +89,94 @@ norm_shift_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __
             const float h0 = xs[0] * wi;
             float acc = h0;
             if (cw != nullptr) {
-                const float* c = cw + (static_cast<int64_t>(sub) * d + i) * taps;
-                acc += c[taps - 1] * h0;
+                const float* c = cw + (static_cast<int64_t>(sub) * taps + taps - 1) * d + i;  // (the newest tap; tap j of a channel lies d floats further a tap)
+                acc += c[0] * h0;
 #pragma unroll
                 for (int m = 1; m < MAXT; ++m) {
-                    if (kind[m] == 1) acc += c[taps - 1 - m] * (xs[m] * wi);
-                    else if (kind[m] == 2) acc += c[taps - 1 - m] * hist[((p - m) % ring) * place + static_cast<int64_t>(sub) * d + i];
+                    if (kind[m] == 1) acc += c[-static_cast<int64_t>(m) * d] * (xs[m] * wi);
+                    else if (kind[m] == 2) acc += c[-static_cast<int64_t>(m) * d] * hist[((p - m) % ring) * place + static_cast<int64_t>(sub) * d + i];
                 }
             }
             out[(static_cast<int64_t>(sub) * n + t) * d + i] = from_float<T>(acc);
             if (hbuf != nullptr) hbuf[static_cast<int64_t>(t) * place + static_cast<int64_t>(sub) * d + i] = h0;
+        }
+    }
+}
+
+// The same for widths that are multiples of four and rows that start at multiples of 16 bytes: a thread takes four channels side
+// by side, so that a row of up to 1,024 channels is one trip to memory a pass, 16 bytes a load, and both sublayers' loads are on
+// their way together. A row's sum of squares is added up in the same order whichever workgroup needs it.
+template <typename T, int MAXT>
+__global__ void __launch_bounds__(kShiftThreads)
+norm_shift_vec_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __restrict__ x, const float* __restrict__ w, float offset, float eps,
+                      const float* __restrict__ cw, int taps, const float* __restrict__ state, int64_t state_stride, int n_slots,
+                      const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ seq_starts,
+                      const int* __restrict__ state_slots, int n, int d, int S) {
+    __shared__ float red[MAXT * (kShiftThreads / kWave)];
+    const int t = blockIdx.x;
+    const int s = tok_seq[t], p = positions[t];
+    const int in_step = t - seq_starts[s];
+    const int ring = taps > 0 ? taps - 1 : 0;
+    int slot = state_slots[s];
+    if (slot < 0 || slot >= n_slots || state == nullptr) slot = -1;
+    int kind[MAXT];  // source m rows back: 1 = a row of the step, 2 = a place of the ring, 0 = nothing
+    float ss[MAXT];
+#pragma unroll
+    for (int m = 0; m < MAXT; ++m) {
+        kind[m] = 0;
+        if (m == 0) kind[m] = 1;
+        else if (m <= ring && p - m >= 0) kind[m] = m <= in_step ? 1 : (slot >= 0 ? 2 : 0);
+        ss[m] = 0.0f;
+    }
+    for (int i = threadIdx.x * 4; i < d; i += kShiftThreads * 4) {
+#pragma unroll
+        for (int m = 0; m < MAXT; ++m) {
+            if (kind[m] == 1) {
+                const f32x4_t v = *reinterpret_cast<const f32x4_t*>(x + static_cast<int64_t>(t - m) * d + i);
+                ss[m] += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+            }
+        }
+    }
+    block_sums<MAXT>(ss, red);
+    float scale[MAXT];
+#pragma unroll
+    for (int m = 0; m < MAXT; ++m) scale[m] = 1.0f / sqrtf(ss[m] / static_cast<float>(d) + eps);
+    const int64_t place = static_cast<int64_t>(S) * d;
+    const float* hist = slot >= 0 ? state + static_cast<int64_t>(slot) * state_stride : nullptr;
+    for (int i = threadIdx.x * 4; i < d; i += kShiftThreads * 4) {
+        f32x4_t xs[MAXT];
+#pragma unroll
+        for (int m = 0; m < MAXT; ++m) {
+            xs[m] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+            if (kind[m] == 1) xs[m] = *reinterpret_cast<const f32x4_t*>(x + static_cast<int64_t>(t - m) * d + i) * scale[m];
+        }
+#pragma unroll
+        for (int sub = 0; sub < kShiftMaxSub; ++sub) {
+            if (sub >= S) break;
+            const f32x4_t wi = *reinterpret_cast<const f32x4_t*>(w + static_cast<int64_t>(sub) * d + i) + offset;
+            const f32x4_t h0 = xs[0] * wi;
+            float acc[4] = {h0[0], h0[1], h0[2], h0[3]};
+            if (cw != nullptr) {
+                const float* c = cw + (static_cast<int64_t>(sub) * taps + taps - 1) * d + i;  // (the newest tap of four channels side by side)
+                const f32x4_t c0 = *reinterpret_cast<const f32x4_t*>(c);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += c0[e] * h0[e];
+#pragma unroll
+                for (int m = 1; m < MAXT; ++m) {
+                    if (kind[m] == 0) continue;
+                    const f32x4_t cm = *reinterpret_cast<const f32x4_t*>(c - static_cast<int64_t>(m) * d);
+                    if (kind[m] == 1) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[e] += cm[e] * (xs[m][e] * wi[e]);
+                    } else {
+                        const f32x4_t hv = *reinterpret_cast<const f32x4_t*>(hist + ((p - m) % ring) * place + static_cast<int64_t>(sub) * d + i);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[e] += cm[e] * hv[e];
+                    }
+                }
+            }
+            store4<T>(out + (static_cast<int64_t>(sub) * n + t) * d + i, acc);
+            if (hbuf != nullptr) *reinterpret_cast<f32x4_t*>(hbuf + static_cast<int64_t>(t) * place + static_cast<int64_t>(sub) * d + i) = h0;
         }
     }
 }
@@ -157,9 +236,17 @@ extern "C" int liyab_norm_shift(void* out, int out_dtype, float* hbuf, const flo
                   "norm_shift: %d taps need the requests' history", taps);
     LIYAB_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "norm_shift: unknown dtype %d", out_dtype);
     if (n == 0) return 0;
+    const auto at16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+    const bool vec = d % 4 == 0 && at16(out) && at16(hbuf) && at16(x) && at16(w) && at16(cw) && (taps <= 1 || (at16(state) && state_stride % 4 == 0));
 #define LIYAB_SHIFT(T, MAXT)                                                                                                                  \
-    norm_shift_kernel<T, MAXT><<<n, kShiftThreads, 0, stream>>>(static_cast<T*>(out), hbuf, x, w, offset, eps, cw, taps, state, state_stride, \
-                                                                  n_slots, tok_seq, positions, seq_starts, state_slots, n, d, S)
+    do { if (vec)                                                                                                                             \
+        norm_shift_vec_kernel<T, MAXT><<<n, kShiftThreads, 0, stream>>>(static_cast<T*>(out), hbuf, x, w, offset, eps, cw, taps, state,      \
+                                                                          state_stride, n_slots, tok_seq, positions, seq_starts, state_slots, \
+                                                                          n, d, S);                                                           \
+    else                                                                                                                                      \
+        norm_shift_kernel<T, MAXT><<<n, kShiftThreads, 0, stream>>>(static_cast<T*>(out), hbuf, x, w, offset, eps, cw, taps, state,          \
+                                                                      state_stride, n_slots, tok_seq, positions, seq_starts, state_slots, n, \
+                                                                      d, S); } while (0)
     if (out_dtype == kF32) {
         if (taps <= 1) LIYAB_SHIFT(float, 1);
         else if (taps <= 4) LIYAB_SHIFT(float, 4);

@@ -1634,7 +1634,7 @@ def norm_shift(out: torch.Tensor, x: torch.Tensor, weights: torch.Tensor, offset
                ring: Optional[StateSlice], ctx, hbuf: Optional[torch.Tensor] = None) -> None:
     """out[s, t] = h_s[t] + sum_j conv[s, :, j] * h_s[t - taps + 1 + j] with h_s = x / sqrt(mean(x^2) + eps) * (weights[s] + offset)
     over each request's own rows in time (conv None: out = h). x float32 [n, d] (the step's rows), weights float32 [S, d],
-    conv float32 [S, d, taps], out [S, n, d] float32 or bfloat16; rows before the step's portion come from `ring` ((taps - 1) x
+    conv float32 [S, taps, d] (a tap's channels side by side), out [S, n, d] float32 or bfloat16; rows before the step's portion come from `ring` ((taps - 1) x
     [S, d] floats, position p at place p % (taps - 1)); `hbuf` float32 [n, S * d] gets h itself, for `ring_keep`."""
     _dev(out, "out")
     _dev(x, "x")
@@ -1648,9 +1648,9 @@ def norm_shift(out: torch.Tensor, x: torch.Tensor, weights: torch.Tensor, offset
     taps = 0
     if conv is not None:
         _dev(conv, "conv")
-        if conv.dtype != torch.float32 or conv.dim() != 3 or tuple(conv.shape[:2]) != (S, d) or not conv.is_contiguous():
-            raise KernelError(f"norm_shift: the convolution's weights must be contiguous float32 [{S}, {d}, taps]")
-        taps = conv.shape[2]
+        if conv.dtype != torch.float32 or conv.dim() != 3 or (conv.shape[0], conv.shape[2]) != (S, d) or not conv.is_contiguous():
+            raise KernelError(f"norm_shift: the convolution's weights must be contiguous float32 [{S}, taps, {d}]")
+        taps = conv.shape[1]
         if not 1 <= taps <= SHIFT_MAX_TAPS:
             raise KernelError(f"norm_shift: {taps} taps; 1 to {SHIFT_MAX_TAPS} are taken")
     if taps > 1 and (ring is None or ring.size != (taps - 1) * S * d):
@@ -1759,7 +1759,7 @@ def maps_store(proj: torch.Tensor, q_out: torch.Tensor, k1: torch.Tensor, k2: to
                conv: Optional[torch.Tensor], ring: Optional[StateSlice], ctx, *, n_head: int, n_kv_head: int, head_dim: int, value_dim: int,
                num_pages: Optional[int] = None) -> None:
     """From a projection's float32 rows [q | k | v] (a query or key head = [map 1 | map 2]) through a causal convolution over time on
-    each channel (conv float32 [C, taps] or None; rows before the step's portion from `ring`, (taps - 1) x [C] floats) to queries
+    each channel (conv float32 [taps, C], a tap's channels side by side, or None; rows before the step's portion from `ring`, (taps - 1) x [C] floats) to queries
     q_out [n, 2, H * P] and keys and values in their slots of the pages (k1, k2, v_cache [pages, G, page_size, P]), zeros behind a
     head's own entries."""
     H, G, D, V = n_head, n_kv_head, head_dim, value_dim
@@ -1779,9 +1779,9 @@ def maps_store(proj: torch.Tensor, q_out: torch.Tensor, k1: torch.Tensor, k2: to
     taps = 0
     if conv is not None:
         _dev(conv, "conv")
-        if conv.dtype != torch.float32 or tuple(conv.shape[:1]) != (C,) or conv.dim() != 2 or not conv.is_contiguous():
-            raise KernelError(f"maps_store: the convolution's weights must be contiguous float32 [{C}, taps]")
-        taps = conv.shape[1]
+        if conv.dtype != torch.float32 or conv.dim() != 2 or conv.shape[1] != C or not conv.is_contiguous():
+            raise KernelError(f"maps_store: the convolution's weights must be contiguous float32 [taps, {C}]")
+        taps = conv.shape[0]
         if not 1 <= taps <= SHIFT_MAX_TAPS:
             raise KernelError(f"maps_store: {taps} taps; 1 to {SHIFT_MAX_TAPS} are taken")
     if taps > 1 and (ring is None or ring.size != (taps - 1) * C):

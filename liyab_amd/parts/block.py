@@ -243,7 +243,8 @@ class ParallelPairBlock:
             if any(c is not None and int(c.taps) != self.taps for c in convs):
                 raise ValueError("a parallel pair's convolutions have one number of taps")
             zero = torch.zeros((self.width, self.taps), dtype=torch.float32, device=self.norm_weights.device)
-            self.conv_weights = torch.stack([c.weight if c is not None else zero for c in convs]).contiguous()
+            # [sublayers, taps, width]: a tap's channels side by side, as the kernel reads them
+            self.conv_weights = torch.stack([c.weight if c is not None else zero for c in convs]).transpose(1, 2).contiguous()
         self.ring_floats = max(self.taps - 1, 0) * self.n_sub * self.width
         own = mixer.state_spec()
         if own is not None and (len(own.shape) != 1 or own.dtype != "float32"):

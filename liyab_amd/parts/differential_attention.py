@@ -55,7 +55,9 @@ class DifferentialAttention:
         if self.taps:
             if not 1 <= self.taps <= ops.SHIFT_MAX_TAPS:
                 raise ValueError(f"a convolution of {self.taps} taps (1 to {ops.SHIFT_MAX_TAPS} are taken)")
-            self.conv = store.fetch_joined([t[c + "_conv"] for c in "qkv"], [(s[0], self.taps) for s in shapes], "vector", "rows")
+            joined = store.fetch_joined([t[c + "_conv"] for c in "qkv"], [(s[0], self.taps) for s in shapes], "vector", "rows")
+            # [taps, channels]: a tap's channels side by side, as the kernel reads them
+            self.conv = store.derived(("taps_major",) + tuple(t[c + "_conv"].name for c in "qkv"), lambda: joined.t().contiguous())
         lam = [store.fetch(t[c], (D,), "vector") for c in ("lq1", "lk1", "lq2", "lk2")]
         self.lam = float(math.exp(float((lam[0].double() * lam[1].double()).sum())) - math.exp(float((lam[2].double() * lam[3].double()).sum()))
                          + float(spec.lam_init))
