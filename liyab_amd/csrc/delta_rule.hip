@@ -166,7 +166,6 @@ delta_scan_kernel(DeltaArgs a) {
         if (more) fetch(c0 + CH);
         const float* buf = lds + which * PER;
         const int n_tok = min(CH, end - c0);
-#pragma unroll 2
         for (int tt = 0; tt < n_tok; ++tt) {
             const float* w = buf + tt * DP + i0;
             const float* au = w + CH * DP;
