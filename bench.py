@@ -488,7 +488,8 @@ def mofulix_prefill_flops(cfg, prompt_lens, logit_rows):
 # The Dopilorn of each size has GPT-2's width, layers, vocabulary and head count; its layers take turns as a delta-rule recurrence
 # (heads of 64, a decay of rank 64), attention in two maps a head (maps of 32, values of 64, as many key heads as query heads, a
 # convolution of four taps on the projections, a window as long as the context, so that each map walks every key) and latent
-# attention (heads of 64 over cached rows of 128, 256 at XL's width, queries through a latent of half the width); two norms and
+# attention (heads of 64 over cached rows of 128, as Bokulix's: the matrix-core kernel for prompts holds rows up to 128; queries through
+# a latent of half the width); two norms and
 # two convolutions of four taps a layer; a feed-forward of two matrices as wide as GPT-2's. It stands beside Mofulix, the engine's
 # other design of parallel layers that mixes recurrences with attention.
 def dopilorn_config(gpt2_cfg):
@@ -499,7 +500,7 @@ def dopilorn_config(gpt2_cfg):
         {"type": "general_delta", "mixer": {"heads": H, "dim": hd, "decay_rank": 64}},
         {"type": "attention", "mixer": {"heads": H, "kv_heads": H, "dim": hd // 2, "vdim": hd, "scale": (hd // 2) ** -0.5, "diff": 0.5, "conv": 4,
                                         "mask": {"size": gpt2_cfg["n_positions"]}}},
-        {"type": "latent_attention", "mixer": {"heads": H, "dim": hd, "vdim": hd, "kv_rank": 256 if d >= 1600 else 128, "q_rank": d // 2 // 64 * 64,
+        {"type": "latent_attention", "mixer": {"heads": H, "dim": hd, "vdim": hd, "kv_rank": 128, "q_rank": d // 2 // 64 * 64,
                                                "scale": hd ** -0.5}},
     ]
     layers = [dict(json.loads(json.dumps(kinds[i % 3])), mlp=dict(mlp)) for i in range(L)]
