@@ -235,11 +235,11 @@ PORTIONS = ((75,), (25, 1, 9, 1, 1, 2, 36), (2,) * 10 + (1,) * 5 + (50,), (1,) *
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width,taps,ff", [(64, 4, 32), (100, 2, None), (72, 1, 24), (96, None, 40), (40, 7, 16), (2500, 3, 8)])
+@pytest.mark.parametrize("width,taps,ff", [(64, 4, 32), (100, 2, None), (72, 1, 24), (96, None, 40), (40, 7, 16), (2500, 3, 8), (66, 3, 20), (50, 5, None)])
 def test_two_norms_and_their_convolutions_in_portions(dtype, width, taps, ff):
     """What the two sublayers read, against the twin: norms with weights stored around zero, the convolutions' history from
     portion to portion down to single tokens, a second request in a slot that was used before, no feed-forward (one sublayer),
-    one tap (no history) and no convolution at all."""
+    one tap (no history) and no convolution at all; widths that are multiples of four (four channels a thread) and not."""
     from liyab_amd.kernels import ops
 
     p = _Layer(dtype, layer("general_delta", delta(1, 8, 2), ff=ff), width=width, taps=taps)
