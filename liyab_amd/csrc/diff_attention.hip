@@ -5,7 +5,8 @@
 //   the same; a value head V values), every channel first through a causal convolution over time when there is one,
 //       y_t = sum_{j < taps} c[j, :] * u_(t - taps + 1 + j)          (zeros before a request's start; c is [taps, C])
 //   whose earlier inputs come from the step's own rows or from the request's history (position p at ring place p % (taps - 1) of
-//   its slot, [C] floats a place, kept by liyab_ring_keep after this kernel has run), to
+//   its slot, [C] floats a place, kept by liyab_ring_keep after this kernel has run, or, with `keep_single`, by this kernel for a
+//   request that brings one token), to
 //     queries  [n, 2, H, P]  (map-major, so that each map is a set of H heads of P for the attention kernels),
 //     keys of map m in plane m of the pages and values in a third plane, all [pages, G, page_size, P],
 //   P >= max(D, V) with zeros behind a head's own entries (zeros add nothing to a score, and nobody reads the values' zeros).
@@ -24,7 +25,8 @@ struct MapsArgs {
     int64_t ld;
     const float* cw;    // [taps, C] or null
     int taps;
-    const float* state; // the ring of slot 0; a slot is state_stride floats further
+    float* state;       // the ring of slot 0; a slot is state_stride floats further
+    int keep_single;    // a request that brings one token keeps its projected row in the ring here (no keeper behind this kernel)
     int64_t state_stride;
     int n_slots;
     void *q_out, *k1, *k2, *vc;
@@ -55,6 +57,8 @@ maps_store_kernel(MapsArgs a) {
         }
     }
     const float* row = a.src + static_cast<int64_t>(t) * a.ld;
+    float* keep = (a.keep_single != 0 && ring > 0 && slot >= 0 && a.seq_starts[s + 1] - a.seq_starts[s] == 1)
+                      ? a.state + static_cast<int64_t>(slot) * a.state_stride + static_cast<int64_t>(p % ring) * C : nullptr;
     const int cache_slot = a.slots[t];
     const bool cached = cache_slot >= 0 && cache_slot < a.num_pages * a.page_size;
     const int page = cached ? cache_slot / a.page_size : 0, off = cached ? cache_slot % a.page_size : 0;
@@ -84,21 +88,23 @@ maps_store_kernel(MapsArgs a) {
             width = V;
             if (cached) dst = static_cast<T*>(a.vc) + ((static_cast<int64_t>(page) * G + g) * a.page_size + off) * P;
         }
-        if (dst == nullptr) continue;
+        if (dst == nullptr && keep == nullptr) continue;
         for (int i = lane; i < P; i += kWave) {
             float acc = 0.0f;
             if (i < width) {
                 const int c = c0 + i;
-                if (a.cw == nullptr) acc = row[c];
+                const float x0 = row[c];
+                if (a.cw == nullptr) acc = x0;
                 else {
                     const float* w = a.cw + static_cast<int64_t>(a.taps - 1) * C + c;  // (the newest tap; a tap's channels lie side by side)
-                    acc = w[0] * row[c];
+                    acc = w[0] * x0;
 #pragma unroll
                     for (int m = 1; m < kMapsMaxTaps; ++m)
                         if (m <= ring && src[m] != nullptr) acc += w[-static_cast<int64_t>(m) * C] * src[m][c];
                 }
+                if (keep != nullptr) keep[c] = x0;  // (the oldest row's place: this thread has just read it)
             }
-            dst[i] = from_float<T>(acc);
+            if (dst != nullptr) dst[i] = from_float<T>(acc);
         }
     }
 }
@@ -128,6 +134,8 @@ maps_store_vec_kernel(MapsArgs a) {
         }
     }
     const float* row = a.src + static_cast<int64_t>(t) * a.ld;
+    float* keep = (a.keep_single != 0 && ring > 0 && slot >= 0 && a.seq_starts[s + 1] - a.seq_starts[s] == 1)
+                      ? a.state + static_cast<int64_t>(slot) * a.state_stride + static_cast<int64_t>(p % ring) * C : nullptr;
     const int cache_slot = a.slots[t];
     const bool cached = cache_slot >= 0 && cache_slot < a.num_pages * a.page_size;
     const int page = cached ? cache_slot / a.page_size : 0, off = cached ? cache_slot % a.page_size : 0;
@@ -148,7 +156,7 @@ maps_store_vec_kernel(MapsArgs a) {
             const int f = c - QC - KC;
             if (cached) dst = paged(a.vc, f / V) + f % V;
         }
-        if (dst != nullptr) {
+        if (dst != nullptr || keep != nullptr) {
             const f32x4 x0 = *reinterpret_cast<const f32x4*>(row + c);
             float acc[4] = {x0[0], x0[1], x0[2], x0[3]};
             if (a.cw != nullptr) {
@@ -165,7 +173,8 @@ maps_store_vec_kernel(MapsArgs a) {
                     }
                 }
             }
-            store4<T>(dst, acc);
+            if (keep != nullptr) *reinterpret_cast<f32x4*>(keep + c) = x0;  // (the oldest row's place: this thread has just read it)
+            if (dst != nullptr) store4<T>(dst, acc);
         }
     }
     // zeros behind the heads' own entries
@@ -211,10 +220,10 @@ maps_join_kernel(T* __restrict__ out, const T* __restrict__ a1, const T* __restr
 
 using namespace liyab;
 
-extern "C" int liyab_maps_store(const float* src, int64_t ld, const float* cw, int taps, const float* state, int64_t state_stride, int n_slots,
+extern "C" int liyab_maps_store(const float* src, int64_t ld, const float* cw, int taps, float* state, int64_t state_stride, int n_slots,
                                 void* q_out, void* k1, void* k2, void* vc, int dtype, const int* slots, int page_size, int num_pages,
                                 const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots, int n, int H, int G,
-                                int D, int V, int P, hipStream_t stream) {
+                                int D, int V, int P, int keep_single, hipStream_t stream) {
     LIYAB_REQUIRE(src && q_out && k1 && k2 && vc && slots && tok_seq && positions && seq_starts && state_slots, "maps_store: null pointer");
     LIYAB_REQUIRE(n >= 0 && H > 0 && G > 0 && D > 0 && V > 0 && P >= D && P >= V && page_size > 0 && num_pages > 0, "maps_store: bad sizes");
     const int64_t C = 2LL * H * D + 2LL * G * D + 1LL * G * V;
@@ -223,7 +232,7 @@ extern "C" int liyab_maps_store(const float* src, int64_t ld, const float* cw, i
     LIYAB_REQUIRE(taps <= 1 || (state != nullptr && n_slots > 0 && state_stride >= (taps - 1) * C), "maps_store: %d taps need the requests' history", taps);
     LIYAB_REQUIRE(dtype == kF32 || dtype == kBF16, "maps_store: unknown dtype %d", dtype);
     if (n == 0) return 0;
-    MapsArgs a{src, ld, cw, taps, state, state_stride, n_slots, q_out, k1, k2, vc, slots, page_size, num_pages, tok_seq, positions, seq_starts,
+    MapsArgs a{src, ld, cw, taps, state, keep_single, state_stride, n_slots, q_out, k1, k2, vc, slots, page_size, num_pages, tok_seq, positions, seq_starts,
                state_slots, H, G, D, V, P};
     const auto at16 = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
     if (D % 4 == 0 && V % 4 == 0 && ld % 4 == 0 && at16(src) && at16(cw) && at16(q_out) && at16(k1) && at16(k2) && at16(vc) &&

@@ -127,8 +127,8 @@ int liyab_attention_scored(void* out, int64_t out_stride, const void* q, int64_t
                            int n_head, int n_kv_head, int dk, int dv, int page_size, int num_pages, hipStream_t stream);
 
 int liyab_norm_shift(void* out, int out_dtype, float* hbuf, const float* x, const float* w, float offset, float eps, const float* cw, int taps,
-                     const float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions, const int* seq_starts,
-                     const int* state_slots, int n, int d, int S, hipStream_t stream);
+                     float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions, const int* seq_starts,
+                     const int* state_slots, int n, int d, int S, int keep_single, hipStream_t stream);
 int liyab_ring_keep(float* state, int64_t state_stride, int ring, int n_slots, const float* src, int64_t ld, int width, const int* tok_seq,
                     const int* positions, const int* context_lens, const int* state_slots, const int* n_real, int n, hipStream_t stream);
 int liyab_normed_powers(void* out, int out_dtype, const float* z, int64_t ld, int n, int ff, const float* coef, float eps, hipStream_t stream);
@@ -141,10 +141,10 @@ int liyab_delta_scan(float* out, const float* r, const float* k, const float* v,
                      int D, int seg_tokens, int max_segs, float* seg_state, float* seg_trans, float* seg_start, hipStream_t stream);
 int liyab_head_norm_gate(void* out, int out_dtype, const float* o, const float* gate, int64_t ldg, const float* w, float eps, int n, int H, int D,
                          hipStream_t stream);
-int liyab_maps_store(const float* src, int64_t ld, const float* cw, int taps, const float* state, int64_t state_stride, int n_slots, void* q_out,
+int liyab_maps_store(const float* src, int64_t ld, const float* cw, int taps, float* state, int64_t state_stride, int n_slots, void* q_out,
                      void* k1, void* k2, void* vc, int dtype, const int* slots, int page_size, int num_pages, const int* tok_seq,
                      const int* positions, const int* seq_starts, const int* state_slots, int n, int H, int G, int D, int V, int P,
-                     hipStream_t stream);
+                     int keep_single, hipStream_t stream);
 int liyab_maps_join(void* out, const void* a1, const void* a2, int64_t lda, int dtype, float lam, float eps, float out_scale, int n, int H, int V,
                     int P, hipStream_t stream);
 

@@ -7,8 +7,9 @@
 // A source row inside the step's portion is normalised again by the workgroup that needs it (the same arithmetic in the
 // same order as its own workgroup's, so the same bits); an earlier one is read, already normalised, from the request's
 // history: position p at ring place p % (taps - 1) of state[slot], each place holding [S, d] floats. `hbuf` [n, S * d]
-// gets h itself for liyab_ring_keep, which runs after every kernel that reads the ring. Everything is 32-bit; the result
-// is rounded once to the output type. Rows behind the step's tokens (position 0 of the first request) read no history.
+// gets h itself for liyab_ring_keep, which runs after every kernel that reads the ring; with `keep_single`, a request that
+// brings one token keeps its row here (a step of single tokens needs no keeper). Everything is 32-bit; the result is rounded
+// once to the output type. Rows behind the step's tokens (position 0 of the first request) read no history.
 //
 // liyab_ring_keep: the last `ring` rows of each request in the step, columns [0, width) of src, go to its history.
 // liyab_normed_powers: out = c1 N(z) + c2 N(z^2) + c3 N(z^3) + c4, N(v) = v / sqrt(mean(v^2) + eps) over a row of z.
@@ -47,9 +48,9 @@ __device__ __forceinline__ void block_sums(float (&v)[COUNT], float* red) {
 template <typename T, int MAXT>
 __global__ void __launch_bounds__(kShiftThreads)
 norm_shift_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __restrict__ x, const float* __restrict__ w, float offset, float eps,
-                  const float* __restrict__ cw, int taps, const float* __restrict__ state, int64_t state_stride, int n_slots,
+                  const float* __restrict__ cw, int taps, float* state, int64_t state_stride, int n_slots,
                   const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ seq_starts,
-                  const int* __restrict__ state_slots, int n, int d, int S) {
+                  const int* __restrict__ state_slots, int n, int d, int S, int keep_single) {
     __shared__ float red[MAXT * (kShiftThreads / kWave)];
     const int t = blockIdx.x;
     const int s = tok_seq[t], p = positions[t];
@@ -79,7 +80,10 @@ norm_shift_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __
 #pragma unroll
     for (int m = 0; m < MAXT; ++m) scale[m] = 1.0f / sqrtf(ss[m] / static_cast<float>(d) + eps);
     const int64_t place = static_cast<int64_t>(S) * d;
-    const float* hist = slot >= 0 ? state + static_cast<int64_t>(slot) * state_stride : nullptr;
+    float* hist = slot >= 0 ? state + static_cast<int64_t>(slot) * state_stride : nullptr;
+    // a request that brings one token: its row takes its place in the ring here (the place of the oldest row, which the same
+    // thread has just read), and no keeper runs behind this kernel
+    const bool keep_own = keep_single != 0 && ring > 0 && slot >= 0 && seq_starts[s + 1] - seq_starts[s] == 1;
     for (int i = threadIdx.x; i < d; i += kShiftThreads) {
         float xs[MAXT];
 #pragma unroll
@@ -99,6 +103,7 @@ norm_shift_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __
             }
             out[(static_cast<int64_t>(sub) * n + t) * d + i] = from_float<T>(acc);
             if (hbuf != nullptr) hbuf[static_cast<int64_t>(t) * place + static_cast<int64_t>(sub) * d + i] = h0;
+            if (keep_own) hist[(p % ring) * place + static_cast<int64_t>(sub) * d + i] = h0;
         }
     }
 }
@@ -109,9 +114,9 @@ norm_shift_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __
 template <typename T, int MAXT>
 __global__ void __launch_bounds__(kShiftThreads)
 norm_shift_vec_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float* __restrict__ x, const float* __restrict__ w, float offset, float eps,
-                      const float* __restrict__ cw, int taps, const float* __restrict__ state, int64_t state_stride, int n_slots,
+                      const float* __restrict__ cw, int taps, float* state, int64_t state_stride, int n_slots,
                       const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ seq_starts,
-                      const int* __restrict__ state_slots, int n, int d, int S) {
+                      const int* __restrict__ state_slots, int n, int d, int S, int keep_single) {
     __shared__ float red[MAXT * (kShiftThreads / kWave)];
     const int t = blockIdx.x;
     const int s = tok_seq[t], p = positions[t];
@@ -142,7 +147,10 @@ norm_shift_vec_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float
 #pragma unroll
     for (int m = 0; m < MAXT; ++m) scale[m] = 1.0f / sqrtf(ss[m] / static_cast<float>(d) + eps);
     const int64_t place = static_cast<int64_t>(S) * d;
-    const float* hist = slot >= 0 ? state + static_cast<int64_t>(slot) * state_stride : nullptr;
+    float* hist = slot >= 0 ? state + static_cast<int64_t>(slot) * state_stride : nullptr;
+    // a request that brings one token: its row takes its place in the ring here (the place of the oldest row, which the same
+    // thread has just read), and no keeper runs behind this kernel
+    const bool keep_own = keep_single != 0 && ring > 0 && slot >= 0 && seq_starts[s + 1] - seq_starts[s] == 1;
     for (int i = threadIdx.x * 4; i < d; i += kShiftThreads * 4) {
         f32x4_t xs[MAXT];
 #pragma unroll
@@ -177,6 +185,7 @@ norm_shift_vec_kernel(T* __restrict__ out, float* __restrict__ hbuf, const float
             }
             store4<T>(out + (static_cast<int64_t>(sub) * n + t) * d + i, acc);
             if (hbuf != nullptr) *reinterpret_cast<f32x4_t*>(hbuf + static_cast<int64_t>(t) * place + static_cast<int64_t>(sub) * d + i) = h0;
+            if (keep_own) *reinterpret_cast<f32x4_t*>(hist + (p % ring) * place + static_cast<int64_t>(sub) * d + i) = h0;
         }
     }
 }
@@ -227,8 +236,8 @@ __global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ p, flo
 using namespace liyab;
 
 extern "C" int liyab_norm_shift(void* out, int out_dtype, float* hbuf, const float* x, const float* w, float offset, float eps, const float* cw,
-                                int taps, const float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions,
-                                const int* seq_starts, const int* state_slots, int n, int d, int S, hipStream_t stream) {
+                                int taps, float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions,
+                                const int* seq_starts, const int* state_slots, int n, int d, int S, int keep_single, hipStream_t stream) {
     LIYAB_REQUIRE(out && x && w && tok_seq && positions && seq_starts && state_slots, "norm_shift: null pointer");
     LIYAB_REQUIRE(n >= 0 && d > 0 && S >= 1 && S <= kShiftMaxSub, "norm_shift: bad sizes n=%d d=%d sublayers=%d", n, d, S);
     LIYAB_REQUIRE(cw == nullptr ? taps == 0 : (taps >= 1 && taps <= kShiftMaxTaps), "norm_shift: %d taps; 1 to %d are taken", taps, kShiftMaxTaps);
@@ -242,11 +251,11 @@ extern "C" int liyab_norm_shift(void* out, int out_dtype, float* hbuf, const flo
     do { if (vec)                                                                                                                             \
         norm_shift_vec_kernel<T, MAXT><<<n, kShiftThreads, 0, stream>>>(static_cast<T*>(out), hbuf, x, w, offset, eps, cw, taps, state,      \
                                                                           state_stride, n_slots, tok_seq, positions, seq_starts, state_slots, \
-                                                                          n, d, S);                                                           \
+                                                                          n, d, S, keep_single);                                              \
     else                                                                                                                                      \
         norm_shift_kernel<T, MAXT><<<n, kShiftThreads, 0, stream>>>(static_cast<T*>(out), hbuf, x, w, offset, eps, cw, taps, state,          \
                                                                       state_stride, n_slots, tok_seq, positions, seq_starts, state_slots, n, \
-                                                                      d, S); } while (0)
+                                                                      d, S, keep_single); } while (0)
     if (out_dtype == kF32) {
         if (taps <= 1) LIYAB_SHIFT(float, 1);
         else if (taps <= 4) LIYAB_SHIFT(float, 4);

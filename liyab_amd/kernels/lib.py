@@ -103,7 +103,7 @@ _SIGNATURES = {
                          c_int, c_float, c_int, P, c_int, P],
     "liyab_attention_scored": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_float, c_int, P, c_int, P, c_int64,
                                c_int, c_int, c_int, c_int, c_int, c_int, P],
-    "liyab_norm_shift": [P, c_int, P, P, P, c_float, c_float, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, c_int, P],
+    "liyab_norm_shift": [P, c_int, P, P, P, c_float, c_float, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, c_int, c_int, P],
     "liyab_ring_keep": [P, c_int64, c_int, c_int, P, c_int64, c_int, P, P, P, P, P, c_int, P],
     "liyab_normed_powers": [P, c_int, P, c_int64, c_int, c_int, P, c_float, P],
     "liyab_softcap": [P, c_float, c_int64, P],
@@ -111,7 +111,7 @@ _SIGNATURES = {
     "liyab_delta_scan": [P, P, P, P, c_int64, P, P, c_int64, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, P],
     "liyab_head_norm_gate": [P, c_int, P, P, c_int64, P, c_float, c_int, c_int, c_int, P],
     "liyab_maps_store": [P, c_int64, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int,
-                         c_int, c_int, c_int, P],
+                         c_int, c_int, c_int, c_int, P],
     "liyab_maps_join": [P, P, P, c_int64, c_int, c_float, c_float, c_float, c_int, c_int, c_int, c_int, P],
 }
 

@@ -1631,11 +1631,13 @@ class StateSlice:
 
 
 def norm_shift(out: torch.Tensor, x: torch.Tensor, weights: torch.Tensor, offset: float, eps: float, conv: Optional[torch.Tensor],
-               ring: Optional[StateSlice], ctx, hbuf: Optional[torch.Tensor] = None) -> None:
+               ring: Optional[StateSlice], ctx, hbuf: Optional[torch.Tensor] = None, keep_single: bool = False) -> None:
     """out[s, t] = h_s[t] + sum_j conv[s, :, j] * h_s[t - taps + 1 + j] with h_s = x / sqrt(mean(x^2) + eps) * (weights[s] + offset)
     over each request's own rows in time (conv None: out = h). x float32 [n, d] (the step's rows), weights float32 [S, d],
     conv float32 [S, taps, d] (a tap's channels side by side), out [S, n, d] float32 or bfloat16; rows before the step's portion come from `ring` ((taps - 1) x
-    [S, d] floats, position p at place p % (taps - 1)); `hbuf` float32 [n, S * d] gets h itself, for `ring_keep`."""
+    [S, d] floats, position p at place p % (taps - 1)); `hbuf` float32 [n, S * d] gets h itself, for `ring_keep`. `keep_single`: a
+    request that brings one token keeps its row in the ring here; a step of single tokens (`single_token_step`) then needs neither
+    `hbuf` nor `ring_keep`."""
     _dev(out, "out")
     _dev(x, "x")
     n, d = x.shape
@@ -1660,7 +1662,14 @@ def norm_shift(out: torch.Tensor, x: torch.Tensor, weights: torch.Tensor, offset
     _step_lists(ctx, n)
     _lib.call("liyab_norm_shift", out.data_ptr(), dtype_code(out.dtype), _ptr(hbuf), x.data_ptr(), weights.data_ptr(), float(offset), float(eps),
               _ptr(conv), taps, ring.data_ptr() if taps > 1 else None, ring.stride if taps > 1 else 0, ring.n_slots if taps > 1 else 0,
-              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, d, S, _stream())
+              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, d, S,
+              1 if keep_single and taps > 1 else 0, _stream())
+
+
+def single_token_step(ctx) -> bool:
+    """Whether every request of the step brings one token (as many rows as requests: it follows from the step's shape, as a
+    captured graph's launches must)."""
+    return ctx.n_tokens == ctx.n_seqs
 
 
 def ring_keep(ring: StateSlice, places: int, src: torch.Tensor, ctx) -> None:
@@ -1757,7 +1766,7 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, wraw: torch.Tensor, w0: to
 # -- attention in two maps a head --------------------------------------------------------------------------------
 def maps_store(proj: torch.Tensor, q_out: torch.Tensor, k1: torch.Tensor, k2: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor,
                conv: Optional[torch.Tensor], ring: Optional[StateSlice], ctx, *, n_head: int, n_kv_head: int, head_dim: int, value_dim: int,
-               num_pages: Optional[int] = None) -> None:
+               num_pages: Optional[int] = None, keep_single: bool = False) -> None:
     """From a projection's float32 rows [q | k | v] (a query or key head = [map 1 | map 2]) through a causal convolution over time on
     each channel (conv float32 [taps, C], a tap's channels side by side, or None; rows before the step's portion from `ring`, (taps - 1) x [C] floats) to queries
     q_out [n, 2, H * P] and keys and values in their slots of the pages (k1, k2, v_cache [pages, G, page_size, P]), zeros behind a
@@ -1791,7 +1800,7 @@ def maps_store(proj: torch.Tensor, q_out: torch.Tensor, k1: torch.Tensor, k2: to
     _lib.call("liyab_maps_store", proj.data_ptr(), ld, _ptr(conv), taps, ring.data_ptr() if taps > 1 else None, ring.stride if taps > 1 else 0,
               ring.n_slots if taps > 1 else 0, q_out.data_ptr(), k1.data_ptr(), k2.data_ptr(), v_cache.data_ptr(), dtype_code(q_out.dtype),
               slots.data_ptr(), k1.shape[2], _pages(k1, num_pages), ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(),
-              ctx.state_slots.data_ptr(), n, H, G, D, V, P, _stream())
+              ctx.state_slots.data_ptr(), n, H, G, D, V, P, 1 if keep_single and taps > 1 else 0, _stream())
 
 
 def maps_join(out: torch.Tensor, a1: torch.Tensor, a2: torch.Tensor, lam: float, eps: float, out_scale: float, *, n_head: int, value_dim: int) -> None:

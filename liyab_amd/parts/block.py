@@ -263,8 +263,10 @@ class ParallelPairBlock:
             ctx.phases.mark(self.mixer_phase)
         ring = ops.StateSlice(state, 0, self.ring_floats) if self.ring_floats else None
         h = ws.get("pair_in", (S, n, d), self.dtype)
-        kept = ws.get("pair_normed", (n, S * d), torch.float32) if ring is not None and writes_cache else None
-        ops.norm_shift(h, x, self.norm_weights, 0.0, self.eps, self.conv_weights, ring, ctx, hbuf=kept)
+        # (a step of single tokens: each row takes its place in the ring inside the kernel that reads the ring)
+        single = ring is not None and writes_cache and ops.single_token_step(ctx)
+        kept = ws.get("pair_normed", (n, S * d), torch.float32) if ring is not None and writes_cache and not single else None
+        ops.norm_shift(h, x, self.norm_weights, 0.0, self.eps, self.conv_weights, ring, ctx, hbuf=kept, keep_single=single)
         # everything that reads the ring has run: the step's last rows take their places in it
         if kept is not None:
             ops.ring_keep(ring, self.taps - 1, kept, ctx)

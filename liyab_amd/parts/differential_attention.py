@@ -82,9 +82,10 @@ class DifferentialAttention:
         ring = own_state(state, (self.taps - 1) * self.channels) if self.taps > 1 else None
         q = ws.get("maps_q", (n, 2, H * P), self.dtype)
         k1, k2, v = cache.rows["k1"], cache.rows["k2"], cache.rows["v"]
+        single = ring is not None and ops.single_token_step(ctx)  # (each row then keeps itself in the ring inside the kernel)
         ops.maps_store(proj, q, k1, k2, v, group.slots, self.conv, ring, ctx, n_head=H, n_kv_head=self.n_kv_head, head_dim=self.head_dim,
-                       value_dim=V)
-        if ring is not None:
+                       value_dim=V, keep_single=single)
+        if ring is not None and not single:
             ops.ring_keep(ring, self.taps - 1, proj, ctx)
         att = ws.get("maps_att", (n, 2, H * P), self.dtype)
         for m, keys in enumerate((k1, k2)):
