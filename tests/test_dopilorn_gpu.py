@@ -589,6 +589,37 @@ def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
         core.manager.check()
 
 
+UNEVEN = {
+    # odd everywhere: width, vocabulary, heads, both head sizes, both latents, the decay's rank, the inner widths
+    "odd": config(577, 77, 1e-6, [layer("general_delta", delta(3, 5, 3), ff=129), layer("attention", maps(3, 1, 5, 7, 0.5, conv=3, window=13), ff=33),
+                                  layer("latent_attention", latent(3, 5, 7, 9, 11), ff=21)], taps=4, cap=15.0, loop=(0, 3, 2)),
+    # even, but no multiple of four (no kernel of four channels a thread takes them), heads of 50
+    "even": config(1001, 250, 1e-5, [layer("attention", maps(5, 5, 10, 14, 0.3, conv=2, window=40), ff=130), layer("general_delta", delta(5, 50, 6), ff=70),
+                                     layer("latent_attention", latent(5, 18, 22, 50, 30), None)], taps=3, loop=(1, 2, 3)),
+    # the widest rows the attention kernels take (cached latents of 256, maps and values of 192) and delta-rule heads of 192
+    "widest": config(512, 128, 1e-5, [layer("latent_attention", latent(2, 96, 96, 256, 64), ff=64), layer("attention", maps(2, 1, 192, 192, 0.5, conv=4, window=100), None),
+                                      layer("general_delta", delta(1, 192, 8), ff=64)], taps=2, cap=30.0),
+}
+
+
+@pytest.mark.parametrize("name", list(UNEVEN))
+def test_sizes_no_kernel_tiles_evenly(name, tmp_path):
+    """Whole prompts and mixed batches at sizes that are odd, even but no multiple of four, and the widest the kernels take."""
+    from liyab_amd.weights import write_random_model
+
+    d = str(tmp_path / "m")
+    write_random_model(d, json.loads(json.dumps(UNEVEN[name])), 7)
+    raw, tensors = read_model(d)
+    reqs = {f"u{i}": tt.random_tokens(70 + i, n, raw["vocab"]) for i, n in enumerate([3, 70, 230])}
+    for dtype in DTYPES:
+        t = twin_tensors(tensors, dtype)
+        ref = {rid: plain.forward(toks, t, raw) for rid, toks in reqs.items()}
+        for steps in (tt.schedule_whole(reqs), tt.schedule_mixed(reqs, seed=1, max_live=3)):
+            core = make_core(d, dtype, None, max_requests=3, num_pages=tt.max_live_pages(steps, 16))
+            check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"dopilorn-uneven {name} {dtype}", family="dopilorn-uneven")
+            core.manager.check()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_real_widths_in_long_steps(dtype, tmp_path):
     """Heads of 64 and 128, a width of 512, prompts of hundreds of tokens in one step and in mixed batches: the tiles of the
