@@ -18,6 +18,7 @@
 //   products, from the unit matrix for P (the product of its A_t); delta_combine_kernel strings a request's segments together
 //   and leaves each the state it starts from; then every segment walks from that state and writes its outputs.
 // liyab_head_norm_gate: out = o / sqrt(mean(o^2 over the head) + eps) * weight * sigmoid(gate), rounded once.
+// liyab_delta_single: all three for a step of single tokens and heads of up to 64, in one kernel.
 #include "common.h"
 #include "launchers.h"
 
@@ -323,6 +324,119 @@ delta_combine_kernel(DeltaArgs a, const float* __restrict__ seg_z, const float* 
     }
 }
 
+// A step in which every request brings one token, heads of up to 64: what liyab_delta_prepare, liyab_delta_scan and
+// liyab_head_norm_gate do in turn, in one kernel, a workgroup a (request, head). The first wave takes the token's decays, rates
+// and unit key and leaves the six vectors in LDS, every wave walks its block of columns for this one token, and the first wave
+// norms and gates the head's result. The arithmetic and its order are those of the three kernels (the same bits).
+struct DeltaSingleArgs {
+    void* out;                // [n, H * D], the compute type
+    const float *r, *k, *v, *araw, *gate;  // rows of ld floats, a head's D values at h * D
+    int64_t ld;
+    const float* wraw;        // rows of ldw floats
+    int64_t ldw;
+    const float *w0, *a_bias, *norm_w;
+    float eps, decay_scale, key_eps;
+    float* state;
+    int64_t state_stride;
+    int n_slots;
+    const int* seq_starts;
+    const int* positions;
+    const int* state_slots;
+    int n_seqs, H, D;
+};
+
+template <typename T, int REG>
+__global__ void __launch_bounds__(kDeltaWaves * kWave)
+delta_single_kernel(DeltaSingleArgs a) {
+    constexpr int DP = 4 * REG;  // 32 or 64
+    static_assert(DP <= kWave, "the first wave holds a head's vectors, an entry a lane");
+    __shared__ __attribute__((aligned(16))) float vec[6 * DP];  // w, a * u, u, k, r, v
+    __shared__ float o_s[kDeltaWaves * kDeltaCols];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int h = blockIdx.x % a.H, s = blockIdx.x / a.H;
+    const int t = a.seq_starts[s];
+    if (a.seq_starts[s + 1] - t != 1) return;  // (the host sends steps of single tokens only)
+    const int D = a.D;
+    if (wave == 0) {
+        const bool in = lane < D;
+        const int64_t at = static_cast<int64_t>(t) * a.ld + h * D + (in ? lane : 0);
+        const int ch = h * D + (in ? lane : 0);
+        const float k = in ? a.k[at] : 0.0f, r = in ? a.r[at] : 0.0f, v = in ? a.v[at] : 0.0f;
+        const float inv = 1.0f / sqrtf(wave_sum(k * k) + a.key_eps);
+        const float u = k * inv;
+        const float w = expf(-a.decay_scale * sigmoid_f(a.wraw[static_cast<int64_t>(t) * a.ldw + ch] + a.w0[ch]));
+        const float rate = sigmoid_f(a.araw[at] + a.a_bias[ch]);
+        if (lane < DP) {
+            vec[lane] = in ? w : 0.0f;
+            vec[DP + lane] = in ? rate * u : 0.0f;
+            vec[2 * DP + lane] = u;
+            vec[3 * DP + lane] = k;
+            vec[4 * DP + lane] = r;
+            vec[5 * DP + lane] = v;
+        }
+    }
+    __syncthreads();
+    const int rb = lane % kDeltaSplit, j = wave * kDeltaCols + lane / kDeltaSplit;
+    const int i0 = rb * REG;
+    const int slot = a.state_slots[s];
+    const bool slot_ok = slot >= 0 && slot < a.n_slots;
+    const bool fresh = a.positions[t] == 0;
+    float* Sg = a.state + static_cast<int64_t>(slot_ok ? slot : 0) * a.state_stride + static_cast<int64_t>(h) * D * D;
+    float S[REG];
+    bool mine[REG];
+#pragma unroll
+    for (int ii = 0; ii < REG; ++ii) {
+        mine[ii] = i0 + ii < D && j < D;
+        S[ii] = (mine[ii] && slot_ok && !fresh) ? Sg[static_cast<int64_t>(i0 + ii) * D + j] : 0.0f;
+    }
+    typedef __attribute__((ext_vector_type(4))) float f32x4;
+    const float* w = vec + i0;
+    const float* au = w + DP;
+    const float* u = au + DP;
+    const float* k = u + DP;
+    const float* r = k + DP;
+    const float v = vec[5 * DP + min(j, DP - 1)];
+    f32x4 seen4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int q4 = 0; q4 < REG / 4; ++q4) {
+        const f32x4 u4 = *reinterpret_cast<const f32x4*>(u + 4 * q4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) seen4[e] += u4[e] * S[4 * q4 + e];
+    }
+    const float seen = group_sum<kDeltaSplit>((seen4[0] + seen4[1]) + (seen4[2] + seen4[3]));
+    f32x4 o4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int q4 = 0; q4 < REG / 4; ++q4) {
+        const f32x4 w4 = *reinterpret_cast<const f32x4*>(w + 4 * q4), a4 = *reinterpret_cast<const f32x4*>(au + 4 * q4);
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(k + 4 * q4), r4 = *reinterpret_cast<const f32x4*>(r + 4 * q4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int ii = 4 * q4 + e;
+            S[ii] = mine[ii] ? w4[e] * S[ii] - a4[e] * seen + k4[e] * v : 0.0f;
+            o4[e] += r4[e] * S[ii];
+        }
+    }
+    const float o = group_sum<kDeltaSplit>((o4[0] + o4[1]) + (o4[2] + o4[3]));
+    if (rb == 0) o_s[j] = j < D ? o : 0.0f;
+    if (slot_ok) {
+#pragma unroll
+        for (int ii = 0; ii < REG; ++ii)
+            if (mine[ii]) Sg[static_cast<int64_t>(i0 + ii) * D + j] = S[ii];
+    }
+    __syncthreads();
+    if (wave == 0) {
+        const bool in = lane < D;
+        const float ov = in ? o_s[lane] : 0.0f;
+        const float scale = 1.0f / sqrtf(wave_sum(ov * ov) / static_cast<float>(D) + a.eps);
+        if (in) {
+            float y = ov * scale;
+            if (a.norm_w != nullptr) y *= a.norm_w[h * D + lane];
+            if (a.gate != nullptr) y *= sigmoid_f(a.gate[static_cast<int64_t>(t) * a.ld + h * D + lane]);
+            static_cast<T*>(a.out)[(static_cast<int64_t>(t) * a.H + h) * D + lane] = from_float<T>(y);
+        }
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_norm_gate_kernel(T* __restrict__ out, const float* __restrict__ o, const float* __restrict__ gate, int64_t ldg, const float* __restrict__ w,
@@ -399,6 +513,32 @@ extern "C" int liyab_delta_scan(float* out, const float* r, const float* k, cons
     }
     walk(a, n_seqs, true);
     return check_launch("delta_scan");
+}
+
+extern "C" int liyab_delta_single_takes(int D) { return D >= 1 && D <= 64 ? 1 : 0; }
+
+extern "C" int liyab_delta_single(void* out, int out_dtype, const float* r, const float* k, const float* v, const float* araw, const float* gate,
+                                  int64_t ld, const float* wraw, int64_t ldw, const float* w0, const float* a_bias, const float* norm_w, float eps,
+                                  float decay_scale, float key_eps, float* state, int64_t state_stride, int n_slots, const int* seq_starts,
+                                  const int* positions, const int* state_slots, int n_seqs, int H, int D, hipStream_t stream) {
+    LIYAB_REQUIRE(out && r && k && v && araw && wraw && w0 && a_bias && state && seq_starts && positions && state_slots, "delta_single: null pointer");
+    LIYAB_REQUIRE(n_seqs >= 0 && H > 0 && liyab_delta_single_takes(D) && ld >= static_cast<int64_t>(H) * D && ldw >= static_cast<int64_t>(H) * D,
+                  "delta_single: bad sizes H=%d D=%d", H, D);
+    LIYAB_REQUIRE(n_slots > 0 && state_stride >= static_cast<int64_t>(H) * D * D, "delta_single: the slot does not hold the heads' matrices");
+    LIYAB_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "delta_single: unknown dtype %d", out_dtype);
+    if (n_seqs == 0) return 0;
+    DeltaSingleArgs a{out, r, k, v, araw, gate, ld, wraw, ldw, w0, a_bias, norm_w, eps, decay_scale, key_eps, state, state_stride, n_slots,
+                      seq_starts, positions, state_slots, n_seqs, H, D};
+    const dim3 grid(static_cast<unsigned>(static_cast<int64_t>(n_seqs) * H));
+    constexpr int T = kDeltaWaves * kWave;
+    if (out_dtype == kF32) {
+        if (D <= 32) delta_single_kernel<float, 8><<<grid, T, 0, stream>>>(a);
+        else delta_single_kernel<float, 16><<<grid, T, 0, stream>>>(a);
+    } else {
+        if (D <= 32) delta_single_kernel<bf16_t, 8><<<grid, T, 0, stream>>>(a);
+        else delta_single_kernel<bf16_t, 16><<<grid, T, 0, stream>>>(a);
+    }
+    return check_launch("delta_single");
 }
 
 extern "C" int liyab_head_norm_gate(void* out, int out_dtype, const float* o, const float* gate, int64_t ldg, const float* w, float eps, int n,

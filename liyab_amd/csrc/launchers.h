@@ -139,6 +139,11 @@ int liyab_delta_prepare(float* prep, const float* k, const float* wraw, const fl
 int liyab_delta_scan(float* out, const float* r, const float* k, const float* v, int64_t ld, const float* prep, float* state,
                      int64_t state_stride, int n_slots, const int* seq_starts, const int* positions, const int* state_slots, int n_seqs, int H,
                      int D, int seg_tokens, int max_segs, float* seg_state, float* seg_trans, float* seg_start, hipStream_t stream);
+int liyab_delta_single_takes(int D);
+int liyab_delta_single(void* out, int out_dtype, const float* r, const float* k, const float* v, const float* araw, const float* gate, int64_t ld,
+                       const float* wraw, int64_t ldw, const float* w0, const float* a_bias, const float* norm_w, float eps, float decay_scale,
+                       float key_eps, float* state, int64_t state_stride, int n_slots, const int* seq_starts, const int* positions,
+                       const int* state_slots, int n_seqs, int H, int D, hipStream_t stream);
 int liyab_head_norm_gate(void* out, int out_dtype, const float* o, const float* gate, int64_t ldg, const float* w, float eps, int n, int H, int D,
                          hipStream_t stream);
 int liyab_maps_store(const float* src, int64_t ld, const float* cw, int taps, float* state, int64_t state_stride, int n_slots, void* q_out,

@@ -117,6 +117,7 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_softcap),
     LIYAB_ENTRY(liyab_delta_prepare),
     LIYAB_ENTRY(liyab_delta_scan),
+    LIYAB_ENTRY(liyab_delta_single),
     LIYAB_ENTRY(liyab_head_norm_gate),
     LIYAB_ENTRY(liyab_maps_store),
     LIYAB_ENTRY(liyab_maps_join),

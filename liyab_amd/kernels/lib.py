@@ -108,6 +108,8 @@ _SIGNATURES = {
     "liyab_normed_powers": [P, c_int, P, c_int64, c_int, c_int, P, c_float, P],
     "liyab_softcap": [P, c_float, c_int64, P],
     "liyab_delta_prepare": [P, P, P, P, c_int64, c_int64, P, P, c_float, c_float, c_int, c_int, c_int, P],
+    "liyab_delta_single": [P, c_int, P, P, P, P, P, c_int64, P, c_int64, P, P, P, c_float, c_float, c_float, P, c_int64, c_int, P, P, P, c_int, c_int,
+                           c_int, P],
     "liyab_delta_scan": [P, P, P, P, c_int64, P, P, c_int64, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, P],
     "liyab_head_norm_gate": [P, c_int, P, P, c_int64, P, c_float, c_int, c_int, c_int, P],
     "liyab_maps_store": [P, c_int64, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int,

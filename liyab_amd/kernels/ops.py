@@ -1713,6 +1713,9 @@ def delta_takes(head_dim: int) -> bool:
     return 1 <= head_dim <= 256
 
 
+DELTA_SINGLE_MAX = 64  # the widest heads the one-kernel form for steps of single tokens takes (csrc/delta_rule.hip)
+
+
 def delta_segments_from(n: int, n_seqs: int) -> bool:
     """Whether a step of n rows of n_seqs requests walks its delta-rule recurrences in segments side by side: when some request
     may bring SCAN_SEGMENT_FROM rows or more. It follows from the step's rows and requests alone (as the grids do), so that a
@@ -1751,10 +1754,17 @@ def delta_rule(out: torch.Tensor, proj: torch.Tensor, wraw: torch.Tensor, w0: to
     if not delta_takes(D) or state.size != H * D * D:
         raise KernelError(f"delta_rule: heads of {D} with {state.size} floats of state a slot")
     _step_lists(ctx, n)
+    p = proj.data_ptr()
+    if single_token_step(ctx) and D <= DELTA_SINGLE_MAX:
+        # every request brings one token: the three kernels' work in one (the same arithmetic in the same order)
+        _lib.call("liyab_delta_single", out.data_ptr(), dtype_code(out.dtype), p, p + 4 * HD, p + 8 * HD, p + 12 * HD, p + 16 * HD, ld,
+                  wraw.data_ptr(), ldw, w0.data_ptr(), a_bias.data_ptr(), _ptr(norm_w), float(eps), float(decay_scale), float(key_eps),
+                  state.data_ptr(), state.stride, state.n_slots, ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(),
+                  ctx.n_seqs, H, D, _stream())
+        return
     ws = ctx.workspace
     prep = ws.get("delta_prep", (n, 3, HD), torch.float32)
     o = ws.get("delta_o", (n, HD), torch.float32)
-    p = proj.data_ptr()
     _lib.call("liyab_delta_prepare", prep.data_ptr(), p + 4 * HD, wraw.data_ptr(), p + 12 * HD, ld, ldw, w0.data_ptr(), a_bias.data_ptr(),
               float(decay_scale), float(key_eps), n, H, D, _stream())
     _lib.call("liyab_delta_scan", o.data_ptr(), p, p + 4 * HD, p + 8 * HD, ld, prep.data_ptr(), state.data_ptr(), state.stride, state.n_slots,
