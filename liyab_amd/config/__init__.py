@@ -28,3 +28,4 @@ from .gpt2 import GPT2Config  # noqa: F401  (registers itself)
 from .bokulix import BokulixConfig  # noqa: F401  (registers itself)
 from .mofulix import MofulixConfig  # noqa: F401  (registers itself)
 from .dopilorn import DopilornConfig  # noqa: F401  (registers itself)
+from .larulorn import LarulornConfig  # noqa: F401  (registers itself)

@@ -128,15 +128,24 @@ class LatentAttentionSpec:
 @dataclass(frozen=True)
 class RoutedFFNSpec:
     """A mixture of gated feed-forward units: each token takes the `top` experts with the largest router
-    logits, weighted by the softmax over those logits alone. Expert: down(act(gate h) * (up h))."""
+    logits, weighted by the softmax over those logits alone. Expert: down(act(gate h) * (up h)).
+    `gated` False: an expert is down(act(up h)) (activation "relu2": the square of the positive part).
+    `groups` = (count, keep): scores are the softmax over all experts; the experts form `count` equal groups of
+    neighbours, a group's score is its largest, and only experts of the `keep` best groups can be chosen; the
+    weights are the chosen scores divided by their sum. `shared_inner` > 0: one more expert of the same form
+    and that inner width runs for every token with weight one (tensors shared_up, shared_down, and shared_gate
+    if gated)."""
 
     kind: str  # "routed_ffn"
     width: int
     inner: int
     n_experts: int
     top: int
-    activation: str  # "silu"
+    activation: str  # "silu" | "relu2"
     tensors: dict = field(default_factory=dict)  # router, router_bias, and per expert e: ("gate", e), ("up", e), ("down", e)
+    gated: bool = True
+    groups: Optional[tuple] = None  # (count, keep)
+    shared_inner: int = 0
 
 
 @dataclass(frozen=True)
@@ -163,11 +172,18 @@ class GateSpec:
 class RotarySpec:
     """Pairs (2i, 2i + 1) of the first `dims` entries of a head turned by position * f_i, f_i = base^(-2i / dims);
     `scaling` (factor, low, high, original) stretches the long wavelengths: f stays where the wavelength is under
-    original / high, becomes f / factor where it is over original / low, and is blended in between."""
+    original / high, becomes f / factor where it is over original / low, and is blended in between.
+    `halves`: the pairs are (i, i + dims / 2) instead. `ramp` (factor, fast, slow, original): the other way of stretching, by the
+    entry's number: with at(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(at(fast)), 0), hi = min(ceil(at(slow)),
+    dims - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), f_i becomes f_i / factor * r_i + f_i (1 - r_i), and cosine and
+    sine are multiplied by `ramp_magnitude` * ln(factor) + 1."""
 
     dims: int
     base: float
     scaling: Optional[tuple] = None  # (factor, low, high, original)
+    halves: bool = False
+    ramp: Optional[tuple] = None  # (factor, fast, slow, original)
+    ramp_magnitude: float = 0.1
 
 
 @dataclass(frozen=True)
@@ -178,7 +194,11 @@ class ScoredAttentionSpec:
     (coef, every): 1 + coef * ln(floor((p + 1) / every) + 1)), a soft cap on the scores (`softcap`: cap * tanh(score / cap)),
     a learned bias by distance (`distance_bias` = the distance from which the table's last row holds; the table's rows:
     the distance itself below half of them, then logarithmic steps), values that are the keys as projected
-    (`values_are_keys`), a sigmoid gate on the heads' results from a projection of the mixer's input (`gated`)."""
+    (`values_are_keys`), a sigmoid gate on the heads' results from a projection of the mixer's input (`gated`), biases on
+    the three projections (`biased`), a learned logit a head that joins the softmax's denominator with no key and no value
+    (`sink`), values shared between layers (`value_mix`: "first" = this layer's values, as projected, are kept for the later
+    layers of the same step; "later" = v <- (1 - lam) v + lam v_first with the learned scalar `vmix`, and the mixed values are
+    what is cached)."""
 
     kind: str  # "scored_attention"
     width: int
@@ -197,7 +217,10 @@ class ScoredAttentionSpec:
     bias_rows: int = 0
     values_are_keys: bool = False
     gated: bool = False
-    tensors: dict = field(default_factory=dict)  # q, k, v, gate, out, q_norm, k_norm, rel
+    tensors: dict = field(default_factory=dict)  # q, k, v, gate, out, q_norm, k_norm, rel, q_bias, k_bias, v_bias, sink, vmix
+    biased: bool = False
+    sink: bool = False
+    value_mix: str = ""  # "" | "first" | "later"
 
 
 @dataclass(frozen=True)
@@ -237,7 +260,8 @@ class StateSpaceSpec:
 @dataclass(frozen=True)
 class SideBySideSpec:
     """Two mixers that read the same input; the result is `weight` times the sum of their results, each brought to unit
-    root mean square over the model's width first and multiplied by a weight of its own."""
+    root mean square over the model's width first and multiplied by a weight of its own. Without `normed`: the results as
+    they are, left_weight * left + right_weight * right, and no tensors."""
 
     kind: str  # "side_by_side"
     width: int
@@ -246,6 +270,25 @@ class SideBySideSpec:
     eps: float
     weight: float = 0.5
     tensors: dict = field(default_factory=dict)  # left_out, right_out
+    normed: bool = True
+    left_weight: float = 1.0
+    right_weight: float = 1.0
+
+
+@dataclass(frozen=True)
+class GatedRecurrenceSpec:
+    """A recurrent block with a linear recurrence a channel under real gates: two branches `inner` wide, y = gelu_tanh(Wy h + by)
+    and u = conv(Wx h + bx) (a causal convolution of `taps` taps a channel with a bias, no activation; its last taps - 1 inputs are
+    part of a request's state); u in `blocks` equal parts, in each r = sigmoid(Ra u + ba) and i = sigmoid(Ri u + bi) with square
+    matrices; a = exp(-rate * r * softplus(lam)); S <- a S + sqrt(1 - a^2) i u from S = 0; the output projection of S * y."""
+
+    kind: str  # "gated_recurrence"
+    width: int
+    inner: int
+    blocks: int
+    taps: int
+    rate: float = 8.0
+    tensors: dict = field(default_factory=dict)  # y, y_bias, x, x_bias, conv, conv_bias, gate_r, gate_r_bias, gate_i, gate_i_bias, lam, out
 
 
 @dataclass(frozen=True)
@@ -339,6 +382,8 @@ class LayerSpec:
     (what the mixer reads is first convolved over time) and the gates are optional.
     arrangement "parallel_pair": x += mixer(c1(norm_mixer(x))) + ffn(c2(norm_ffn(x))): two norms of the same x, each
     followed by a convolution over time of its own (`input_conv`, `ffn_conv`: h <- h + conv(h); optional).
+    arrangement "sandwich": x += post_norm_mixer(mixer(norm_mixer(x))); x += post_norm_ffn(ffn(norm_ffn(x))): a norm before and
+    a norm behind each sublayer.
     `entry`: what is done to the stream before the layer runs (a spec of the entry registry), or None.
     """
 
@@ -352,6 +397,8 @@ class LayerSpec:
     gate_ffn: Any = None
     ffn_conv: Any = None
     entry: Any = None
+    post_norm_mixer: Any = None
+    post_norm_ffn: Any = None
 
 
 @dataclass(frozen=True)

@@ -70,9 +70,21 @@ __device__ __forceinline__ void merge_partial(Partial& a, float mo, float lo, co
     a.m = M;
 }
 
+// A sink joins a row's softmax: a learned logit a head that stands in the denominator once, as a key would whose score it is,
+// and has no value. (m, l, acc): the row's maximum, sum and weighted values, rescaled to the larger of m and the sink.
+template <typename T, int N = 8>
+__device__ __forceinline__ void add_sink(float& m, float& l, float (&acc)[N], float sink) {
+    const float M = fmaxf(m, sink);
+    const float w = m == -INFINITY ? 0.0f : exp_for<T>(m - M);
+    l = l * w + exp_for<T>(sink - M);
+#pragma unroll
+    for (int e = 0; e < N; ++e) acc[e] *= w;
+    m = M;
+}
+
 // SCORED: the score scale * q . k is worked on before the softmax: a soft cap, cap * tanh(score / cap) (softcap > 0), then
-// a bias by distance, bias_table[min(position - key, max_dist), head] (bias_table given). Without SCORED the three
-// arguments are not read, and the kernel is the one it was.
+// a bias by distance, bias_table[min(position - key, max_dist), head] (bias_table given); `sinks` (one logit a head) join the
+// softmax's denominator where the row's sums are final. Without SCORED these arguments are not read, and the kernel is the one it was.
 template <typename T, int LPK, int AD_WAVES, int AD_U, bool SCORED = false>
 __global__ void __launch_bounds__(64 * AD_WAVES)
 attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ q, int64_t q_stride,
@@ -81,7 +93,7 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
                         const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, float scale, int window,
                         int n_head, int n_kv_head, int hd, int page_size, int page_shift, int rows_are_requests,
                         int n_splits, int chunk, float* __restrict__ partials, int num_pages, float softcap = 0.0f,
-                        const float* __restrict__ bias_table = nullptr, int max_dist = 0) {
+                        const float* __restrict__ bias_table = nullptr, int max_dist = 0, const float* __restrict__ sinks = nullptr) {
     constexpr int KPP = 64 / LPK;  // keys per wave and pass
     __shared__ float lds2[2][AD_WAVES][LPK][10];  // the waves' sums, for the first wave to merge; two of them in turn, so that one barrier a split is enough
     const int t = tok_list != nullptr ? tok_list[blockIdx.x] : blockIdx.x;
@@ -211,6 +223,9 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
             for (int e = 0; e < 8; ++e) stash[zi][c][2 + e] = st.acc[e];
         } else if (n_splits == 1) {
             T* o = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
+            if constexpr (SCORED) {
+                if (sinks != nullptr) add_sink<T>(st.m, st.l, st.acc, sinks[h]);
+            }
             if (chunk > 0) {
                 // as the merge of several splits divides: a token has the same bits alone in one split
                 // and beside longer contexts, its later splits empty
@@ -249,6 +264,9 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
 #pragma unroll
             for (int e = 0; e < 8; ++e) o[e] = fmaf(w, stash[zi][c][2 + e], o[e]);
         }
+        if constexpr (SCORED) {
+            if (sinks != nullptr) add_sink<T>(M, sum, o, sinks[h]);
+        }
         T* dst = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + c * 8;
 #pragma unroll
         for (int e = 0; e < 8; ++e) dst[e] = from_float<T>(o[e] / sum);
@@ -258,7 +276,8 @@ attention_decode_kernel(T* __restrict__ out, int64_t out_stride, const T* __rest
 // Splits of a (token, head) merged in split order (the same operations as the end of the kernel above).
 template <typename T>
 __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, const int* __restrict__ tok_list,
-                                       const float* __restrict__ partials, int n_head, int hd, int n_splits) {
+                                       const float* __restrict__ partials, int n_head, int hd, int n_splits,
+                                       const float* __restrict__ sinks = nullptr) {
     // The splits' maxima and sums go to LDS first, a lane a split, and the values are fetched
     // eight splits at a time before they are used: the sums below are one chain in split order,
     // and a load at a time inside it would cost its latency once a split.
@@ -294,6 +313,11 @@ __global__ void attention_merge_kernel(T* __restrict__ out, int64_t out_stride, 
             o = fmaf(w, a[u], o);
         }
     }
+    if (sinks != nullptr) {
+        float one[1] = {o};
+        add_sink<T, 1>(M, sum, one, sinks[h]);
+        o = one[0];
+    }
     out[static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * hd + e] = from_float<T>(o / sum);
 }
 
@@ -303,7 +327,7 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
                             const int* tok_pos, int n, float scale, int window, int n_head, int n_kv_head, int hd,
                             int page_size, int n_splits, int chunk, int waves, int rows_are_requests, float* partials,
                             int leave_splits, int num_pages, hipStream_t stream, float softcap = 0.0f, const float* bias_table = nullptr,
-                            int max_dist = 0) {
+                            int max_dist = 0, const float* sinks = nullptr) {
     int page_shift = -1;
     for (int b = 0; b < 31; ++b)
         if ((1 << b) == page_size) page_shift = b;
@@ -317,15 +341,15 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
         if (waves == 4)                                                                                              \
             attention_decode_kernel<T, L, 4, 4, SCORED><<<grid, 256, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist, sinks); \
         else if (waves == 8)                                                                                         \
             attention_decode_kernel<T, L, 8, 4, SCORED><<<grid, 512, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                     max_blocks, tok_list, tok_seq, tok_pos, scale,   \
-                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist); \
+                                                                    window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist, sinks); \
         else                                                                                                         \
             attention_decode_kernel<T, L, 16, sizeof(T) == 2 ? 8 : 4, SCORED><<<grid, 1024, 0, stream>>>(o, out_stride, pq, q_stride, pk, pv, block_tables, \
                                                                       max_blocks, tok_list, tok_seq, tok_pos, scale, \
-                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist); \
+                                                                      window, n_head, n_kv_head, hd, page_size, page_shift, rows_are_requests, n_splits, chunk, partials, num_pages, softcap, bias_table, max_dist, sinks); \
     } while (0)
     if (hd <= 8) LIYAB_GO(1);
     else if (hd <= 16) LIYAB_GO(2);
@@ -336,7 +360,7 @@ int launch_attention_decode(void* out, int64_t out_stride, const void* q, int64_
 #undef LIYAB_GO
     if (int rc = check_launch("attention_decode")) return rc;
     if (n_splits > 1 && !leave_splits) {
-        attention_merge_kernel<T><<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(o, out_stride, tok_list, partials, n_head, hd, n_splits);
+        attention_merge_kernel<T><<<dim3(n, n_head), ((hd + 63) / 64) * 64, 0, stream>>>(o, out_stride, tok_list, partials, n_head, hd, n_splits, sinks);
         return check_launch("attention_merge");
     }
     return 0;
@@ -404,25 +428,27 @@ extern "C" int liyab_attention_decode(void* out, int64_t out_stride, const void*
 }
 
 // The same with the scores worked on before the softmax: softcap > 0 caps them, cap * tanh(score / cap); bias_table (float
-// [max_dist + 1, n_head]) adds table[min(position - key, max_dist), head].
+// [max_dist + 1, n_head]) adds table[min(position - key, max_dist), head]; sinks (float [n_head], or null): exp(sinks[head])
+// is added to the softmax's denominator.
 extern "C" int liyab_attention_decode_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                              const void* vc, int dtype, const int* block_tables, int max_blocks, const int* tok_list,
                                              const int* tok_seq, const int* tok_pos, int n, float scale, int window,
                                              int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk, int waves,
                                              int rows_are_requests, float* partials, int leave_splits, int num_pages, float softcap,
-                                             const float* bias_table, int max_dist, hipStream_t stream) {
+                                             const float* bias_table, int max_dist, const float* sinks, hipStream_t stream) {
     if (int rc = check_attention_decode(out, out_stride, q, q_stride, kc, vc, dtype, block_tables, max_blocks, tok_list, tok_seq, tok_pos, n, window,
                                         n_head, n_kv_head, hd, page_size, n_splits, chunk, waves, rows_are_requests, partials, leave_splits, num_pages))
         return rc;
     LIYAB_REQUIRE(softcap >= 0.0f && (bias_table == nullptr || max_dist >= 0), "attention_decode_scored: a negative cap or distance");
+    LIYAB_REQUIRE(sinks == nullptr || !leave_splits, "attention_decode_scored: splits left unmerged take no sink");
     if (n == 0) return 0;
     if (dtype == kF32)
         return launch_attention_decode<float, true>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
                                                     tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
-                                                    rows_are_requests, partials, leave_splits, num_pages, stream, softcap, bias_table, max_dist);
+                                                    rows_are_requests, partials, leave_splits, num_pages, stream, softcap, bias_table, max_dist, sinks);
     return launch_attention_decode<bf16_t, true>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, tok_list, tok_seq,
                                                  tok_pos, n, scale, window, n_head, n_kv_head, hd, page_size, n_splits, chunk, waves,
-                                                 rows_are_requests, partials, leave_splits, num_pages, stream, softcap, bias_table, max_dist);
+                                                 rows_are_requests, partials, leave_splits, num_pages, stream, softcap, bias_table, max_dist, sinks);
 }
 
 // out[m, h * hd + e] = the splits of (m, h) merged in split order: for splits that

@@ -61,14 +61,16 @@ constexpr int AP_MAX_BLOCKS = 2048;  // page ids of a tile's keys are kept in LD
 
 // SCORED: the scores are worked on before the softmax: scale * q . k, capped as cap * tanh(. / cap) when softcap > 0, plus
 // bias_table[min(query position - key position, max_dist), head] when a table is given; the exponentials then take the
-// scores as they are. Without SCORED the three arguments are not read, and the kernel is the one it was.
+// scores as they are; `sinks` (one logit a head) join the denominator once the row's sums are final. Without SCORED these
+// arguments are not read, and the kernel is the one it was.
 template <int DB, int QG, int KS, int NS = 1, bool SCORED = false>  // head dimension padded to 32 * DB; 32 * QG queries a tile; KS x NS blocks of keys a step, NS a wave
 __global__ void __launch_bounds__(64 * QG * KS)
 attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
                          const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ work, float scale,
                          int window, int n_head, int n_kv_head, int hd, int page_size, int page_shift, int num_pages,
-                         float softcap = 0.0f, const float* __restrict__ bias_table = nullptr, int max_dist = 0) {
+                         float softcap = 0.0f, const float* __restrict__ bias_table = nullptr, int max_dist = 0,
+                         const float* __restrict__ sinks = nullptr) {
     constexpr int HDP = 32 * DB;
     constexpr int LDK = HDP + 8;  // padded row: 16-byte reads of 16 lanes fall in distinct banks
     constexpr int WAVES = QG * KS, THREADS = 64 * WAVES;
@@ -378,7 +380,16 @@ attention_prefill_kernel(bf16_t* __restrict__ out, int64_t out_stride, const bf1
     // o[d][r] = O^T[dim = 32 d + 8 (r / 4) + 4 g2 + r % 4][query ql]: through LDS to rows of 16-byte pieces
     const bool writes = wave_has && ks == 0;
     if (writes) {
-        const float inv = 1.0f / l_run;
+        float inv = 1.0f / l_run;
+        if constexpr (SCORED) {
+            if (sinks != nullptr) {
+                // a sink: one more term of the denominator, exp(sink) against the row's reference (both in powers of two)
+                const float s2 = sinks[h] * 1.4426950408889634f;
+                const float M = fmaxf(m_run, s2);
+                const float w = m_run == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run - M);
+                inv = w / (l_run * w + __builtin_amdgcn_exp2f(s2 - M));
+            }
+        }
 #pragma unroll
         for (int d = 0; d < DB; ++d)
 #pragma unroll
@@ -410,7 +421,8 @@ template <bool SCORED>
 static int run_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                  const void* vc, const int* block_tables, int max_blocks, const int* work,
                                  int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
-                                 int page_size, int num_pages, float softcap, const float* bias_table, int max_dist, hipStream_t stream) {
+                                 int page_size, int num_pages, float softcap, const float* bias_table, int max_dist, const float* sinks,
+                                 hipStream_t stream) {
     LIYAB_REQUIRE(out && q && kc && vc && block_tables && work, "attention_prefill: null pointer");
     LIYAB_REQUIRE(num_pages > 0, "attention_prefill: the caches hold %d pages", num_pages);
     LIYAB_REQUIRE(n_tiles >= 0 && n_head > 0 && n_kv_head > 0 && page_size > 0 && max_blocks > 0, "attention_prefill: bad sizes");
@@ -439,7 +451,7 @@ static int run_attention_prefill(void* out, int64_t out_stride, const void* q, i
     auto* pv = static_cast<const bf16_t*>(vc);
 #define LIYAB_RUN(D, Q, S)                                                                                          \
     attention_prefill_kernel<D, Q, S, (D <= 2 && Q == 4 && S <= 2) ? 2 : 1, SCORED><<<grid, 64 * Q * S, 0, stream>>>(                          \
-        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift, num_pages, softcap, bias_table, max_dist)
+        o, out_stride, pq, q_stride, pk, pv, block_tables, max_blocks, work, scale, window, n_head, n_kv_head, hd, page_size, page_shift, num_pages, softcap, bias_table, max_dist, sinks)
 #define LIYAB_RUN4(D) LIYAB_RUN(D, 2, 4)
 #define LIYAB_SKIP4(D) (void)0  // four stages of 128 keys do not fit LDS at these head sizes (refused above)
 #define LIYAB_GO(D, FOUR)                           \
@@ -469,17 +481,18 @@ extern "C" int liyab_attention_prefill(void* out, int64_t out_stride, const void
                                        int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
                                        int page_size, int num_pages, hipStream_t stream) {
     return run_attention_prefill<false>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, work, n_tiles, tile, ksplit, scale, window,
-                                        n_head, n_kv_head, hd, page_size, num_pages, 0.0f, nullptr, 0, stream);
+                                        n_head, n_kv_head, hd, page_size, num_pages, 0.0f, nullptr, 0, nullptr, stream);
 }
 
 // The same with the scores worked on before the softmax: softcap > 0 caps them, cap * tanh(score / cap); bias_table (float
-// [max_dist + 1, n_head]) adds table[min(query position - key position, max_dist), head].
+// [max_dist + 1, n_head]) adds table[min(query position - key position, max_dist), head]; sinks (float [n_head], or null):
+// exp(sinks[head]) is added to the softmax's denominator.
 extern "C" int liyab_attention_prefill_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc,
                                               const void* vc, const int* block_tables, int max_blocks, const int* work,
                                               int n_tiles, int tile, int ksplit, float scale, int window, int n_head, int n_kv_head, int hd,
                                               int page_size, int num_pages, float softcap, const float* bias_table, int max_dist,
-                                              hipStream_t stream) {
+                                              const float* sinks, hipStream_t stream) {
     LIYAB_REQUIRE(softcap >= 0.0f && (bias_table == nullptr || max_dist >= 0), "attention_prefill_scored: a negative cap or distance");
     return run_attention_prefill<true>(out, out_stride, q, q_stride, kc, vc, block_tables, max_blocks, work, n_tiles, tile, ksplit, scale, window,
-                                       n_head, n_kv_head, hd, page_size, num_pages, softcap, bias_table, max_dist, stream);
+                                       n_head, n_kv_head, hd, page_size, num_pages, softcap, bias_table, max_dist, sinks, stream);
 }

@@ -8,12 +8,14 @@
 // they meet: g = min(G, limit), u = clamp(U, -limit, limit), y = g * sigmoid(slope * g) * (u + shift),
 // from one 32-bit product [G | U] a row.
 //
-// liyab_activate: tanh, silu or the logistic function of 32-bit rows, rounded to the output type.
+// liyab_activate: tanh, silu, the logistic function or the squared positive part of 32-bit rows, rounded to the output type.
 //
 // liyab_gate_rows: x *= sigmoid(g) in place, a gate on a mixer's rows from 32-bit logits.
 //
 // liyab_mean_norm_add: x += weight * (a / rms(a) * wa + b / rms(b) * wb), the two results of
 // sublayers that run side by side, each brought to unit root mean square over the row first.
+//
+// liyab_weighted_sum: out = wa * a + wb * b, two sublayers' results joined with constant weights.
 //
 // All arithmetic is 32-bit; a result is rounded once, to the output type.
 #include "common.h"
@@ -61,7 +63,7 @@ activate_kernel(T* __restrict__ out, int64_t ldo, const float* __restrict__ in, 
     const int i = blockIdx.x * EW_THREADS + threadIdx.x;
     if (i >= d) return;
     const float z = in[static_cast<int64_t>(t) * ldi + i];
-    const float v = op == 0 ? tanhf(z) : op == 1 ? z * logistic(z) : logistic(z);
+    const float v = op == 0 ? tanhf(z) : op == 1 ? z * logistic(z) : op == 2 ? logistic(z) : (z > 0.0f ? z * z : 0.0f);
     out[static_cast<int64_t>(t) * ldo + i] = from_float<T>(v);
 }
 
@@ -103,9 +105,23 @@ mean_norm_add_kernel(float* __restrict__ x, const float* __restrict__ a, const f
         x[row + i] += weight * (a[row + i] * ra * wa[i] + b[row + i] * rb * wb[i]);
 }
 
+__global__ void __launch_bounds__(EW_THREADS)
+weighted_sum_kernel(float* __restrict__ out, const float* __restrict__ a, const float* __restrict__ b, float wa, float wb, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * EW_THREADS + threadIdx.x;
+    if (i < n) out[i] = wa * a[i] + wb * b[i];
+}
+
 }  // namespace liyab
 
 using namespace liyab;
+
+extern "C" int liyab_weighted_sum(float* out, const float* a, const float* b, float wa, float wb, int64_t n, hipStream_t stream) {
+    LIYAB_REQUIRE(out && a && b, "weighted_sum: null pointer");
+    LIYAB_REQUIRE(n >= 0 && n < (int64_t(1) << 38), "weighted_sum: bad size");
+    if (n == 0) return 0;
+    weighted_sum_kernel<<<static_cast<unsigned>((n + EW_THREADS - 1) / EW_THREADS), EW_THREADS, 0, stream>>>(out, a, b, wa, wb, n);
+    return check_launch("weighted_sum");
+}
 
 extern "C" int liyab_dyt(void* out, int out_dtype, const float* x, const float* w, const float* b, const float* alpha, const int* rows,
                          int n, int d, hipStream_t stream) {
@@ -134,7 +150,7 @@ extern "C" int liyab_glu_clamped(void* out, int out_dtype, const float* gu, int6
 extern "C" int liyab_activate(void* out, int out_dtype, int64_t ldo, const float* in, int64_t ldi, int op, int n, int d, hipStream_t stream) {
     LIYAB_REQUIRE(out && in, "activate: null pointer");
     LIYAB_REQUIRE(n >= 0 && n <= 65535 && d > 0 && ldo >= d && ldi >= d, "activate: bad sizes");
-    LIYAB_REQUIRE(op >= 0 && op <= 2, "activate: unknown function %d", op);
+    LIYAB_REQUIRE(op >= 0 && op <= 3, "activate: unknown function %d", op);
     if (n == 0) return 0;
     dim3 grid((d + EW_THREADS - 1) / EW_THREADS, n);
     if (out_dtype == kF32) activate_kernel<float><<<grid, EW_THREADS, 0, stream>>>(static_cast<float*>(out), ldo, in, ldi, op, d);

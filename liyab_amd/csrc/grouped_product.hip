@@ -6,8 +6,8 @@
 //   a row = a + (idx / a_div) * lda + g * a_group_cols       (a_div: entries a token, so that a
 //                                                             token's row serves each of its experts)
 //   w[g]  = w + g * N * K, a row an output feature ([N, K], K contiguous)
-//   out   = out + idx * ldo + g * out_group_cols + column
-//   value = acc0                                 (one matrix)
+//   out   = out + (idx + (idx / out_div) * out_extra) * ldo + g * out_group_cols + column
+//   value = acc0, or relu(acc0)^2 with act = 1   (one matrix)
 //         = silu(acc0) * acc1                    (two matrices: a gated unit's first products)
 //     then * row_scale[idx] (a router's weight), * sigmoid(gate[idx * gate_stride + g * N + column])
 //     (the gate's logits float32 or bfloat16)
@@ -41,6 +41,8 @@ struct GroupedParams {
     int gate_dtype;
     int M, N, K;
     int block;  // places a tile of rows_list: kGroupedRows, or kSkinnyRows for steps of few rows
+    int act;        // one matrix: 0 = the sums as they are, 1 = the square of their positive part (relu(.)^2)
+    int out_div, out_extra;  // `out_extra` rows of `out` are left free behind each `out_div` rows (a token's entries), for results another product adds
 };
 
 __device__ __forceinline__ float gp_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
@@ -49,12 +51,13 @@ template <int NW>
 __device__ __forceinline__ void grouped_store(const GroupedParams& p, int idx, int g, int n, float v0, float v1) {
     float v = v0;
     if constexpr (NW == 2) v = v0 * gp_sigmoid(v0) * v1;
+    else if (p.act == 1) v = v0 > 0.0f ? v0 * v0 : 0.0f;
     if (p.row_scale != nullptr) v *= p.row_scale[idx];
     if (p.gate != nullptr) {
         const int64_t ga = static_cast<int64_t>(idx) * p.gate_stride + static_cast<int64_t>(g) * p.N + n;
         v *= gp_sigmoid(p.gate_dtype == kF32 ? static_cast<const float*>(p.gate)[ga] : bf16_to_float(static_cast<const bf16_t*>(p.gate)[ga]));
     }
-    const int64_t at = static_cast<int64_t>(idx) * p.ldo + static_cast<int64_t>(g) * p.out_group_cols + n;
+    const int64_t at = static_cast<int64_t>(idx + (idx / p.out_div) * p.out_extra) * p.ldo + static_cast<int64_t>(g) * p.out_group_cols + n;
     if (p.out_dtype == kF32)
         static_cast<float*>(p.out)[at] = v;
     else
@@ -353,7 +356,8 @@ using namespace liyab;
 extern "C" int liyab_grouped_product(const void* a, int64_t lda, int a_div, int a_group_cols, const void* w0, const void* w1, int dtype,
                                      void* out, int out_dtype, int64_t ldo, int out_group_cols, const int* rows_list,
                                      const int* tile_group, int n_tiles, int block, int n_groups, const float* row_scale,
-                                     const void* gate, int gate_dtype, int64_t gate_stride, int M, int N, int K, hipStream_t stream) {
+                                     const void* gate, int gate_dtype, int64_t gate_stride, int M, int N, int K, int act, int out_div, int out_extra,
+                                     hipStream_t stream) {
     LIYAB_REQUIRE(a && w0 && out, "grouped_product: null pointer");
     LIYAB_REQUIRE(dtype == kF32 || dtype == kBF16, "grouped_product: unknown dtype %d", dtype);
     LIYAB_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "grouped_product: unknown output dtype %d", out_dtype);
@@ -363,8 +367,9 @@ extern "C" int liyab_grouped_product(const void* a, int64_t lda, int a_div, int 
     LIYAB_REQUIRE(rows_list != nullptr || n_tiles == (M + block - 1) / block, "grouped_product: %d tiles for %d rows", n_tiles, M);
     LIYAB_REQUIRE(gate == nullptr || gate_dtype == kF32 || gate_dtype == kBF16, "grouped_product: unknown gate dtype %d", gate_dtype);
     LIYAB_REQUIRE(gate == nullptr || gate_stride >= static_cast<int64_t>(rows_list ? 1 : n_groups) * N, "grouped_product: the gate's rows are shorter than the output's");
+    LIYAB_REQUIRE((act == 0 || (act == 1 && w1 == nullptr)) && out_div >= 1 && out_extra >= 0, "grouped_product: unknown activation %d, or one beside a gated unit", act);
     if (M == 0 || n_tiles == 0) return 0;
-    GroupedParams p{a, lda, a_div, a_group_cols, w0, w1, out, ldo, out_group_cols, out_dtype, rows_list, tile_group, row_scale, gate, gate_stride, gate_dtype, M, N, K, block};
+    GroupedParams p{a, lda, a_div, a_group_cols, w0, w1, out, ldo, out_group_cols, out_dtype, rows_list, tile_group, row_scale, gate, gate_stride, gate_dtype, M, N, K, block, act, out_div, out_extra};
     const dim3 grid(n_tiles, (N + 63) / 64, rows_list ? 1 : n_groups);
     const bool matrix = dtype == kBF16 && K % 8 == 0 && lda % 8 == 0 && a_group_cols % 8 == 0 &&
                         (reinterpret_cast<uintptr_t>(a) & 15) == 0 && (reinterpret_cast<uintptr_t>(w0) & 15) == 0 &&

@@ -74,10 +74,11 @@ int liyab_latent_store(void* cache, int dtype, const void* src, int64_t src_stri
 int liyab_grouped_product(const void* a, int64_t lda, int a_div, int a_group_cols, const void* w0, const void* w1, int dtype, void* out,
                           int out_dtype, int64_t ldo, int out_group_cols, const int* rows_list, const int* tile_group, int n_tiles,
                           int block, int n_groups, const float* row_scale, const void* gate, int gate_dtype, int64_t gate_stride, int M, int N,
-                          int K, hipStream_t stream);
-int liyab_moe_route(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, hipStream_t stream);
+                          int K, int act, int out_div, int out_extra, hipStream_t stream);
+int liyab_moe_route(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, int mode, int n_groups, int keep,
+                    hipStream_t stream);
 int liyab_moe_route_align(const float* logits, int64_t ld, int n, int n_experts, int top, int* ids, float* weights, int block,
-                          int* rows_list, int* tile_group, int max_tiles, hipStream_t stream);
+                          int* rows_list, int* tile_group, int max_tiles, int mode, int n_groups, int keep, hipStream_t stream);
 int liyab_moe_align(const int* ids, int n_entries, int n_experts, int block, int* rows_list, int* tile_group, int max_tiles,
                     hipStream_t stream);
 
@@ -85,11 +86,11 @@ int liyab_attention_decode_scored(void* out, int64_t out_stride, const void* q, 
                                   const int* block_tables, int max_blocks, const int* tok_list, const int* tok_seq, const int* tok_pos, int n,
                                   float scale, int window, int n_head, int n_kv_head, int hd, int page_size, int n_splits, int chunk,
                                   int waves, int rows_are_requests, float* partials, int leave_splits, int num_pages, float softcap,
-                                  const float* bias_table, int max_dist, hipStream_t stream);
+                                  const float* bias_table, int max_dist, const float* sinks, hipStream_t stream);
 int liyab_attention_prefill_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc,
                                    const int* block_tables, int max_blocks, const int* work, int n_tiles, int tile, int ksplit, float scale,
                                    int window, int n_head, int n_kv_head, int hd, int page_size, int num_pages, float softcap,
-                                   const float* bias_table, int max_dist, hipStream_t stream);
+                                   const float* bias_table, int max_dist, const float* sinks, hipStream_t stream);
 int liyab_gate_rows(void* x, int dtype, int64_t ldx, const float* gate, int64_t ldg, int n, int d, hipStream_t stream);
 int liyab_dyt(void* out, int out_dtype, const float* x, const float* w, const float* b, const float* alpha, const int* rows, int n, int d,
               hipStream_t stream);
@@ -114,17 +115,17 @@ int liyab_token_shift(void* out, int dtype, const void* h, const float* mu, int 
                       hipStream_t stream);
 int liyab_conv_act(float* out, int64_t ldo, const float* in, int64_t ldi, const float* w, const float* bias, int taps, const float* state,
                    int64_t state_stride, int n_slots, const int* tok_seq, const int* positions, const int* seq_starts,
-                   const int* state_slots, int n, int C, hipStream_t stream);
+                   const int* state_slots, int n, int C, int act, hipStream_t stream);
 int liyab_gated_group_norm(void* out, int out_dtype, const float* y, int64_t ldy, const float* z, int64_t ldz, const float* w, float eps,
                            int n, int inner, int groups, hipStream_t stream);
 int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, int dk_out, int dv_out,
                      void* q_out, void* kc, void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm, const float* k_norm,
                      float eps, const float* freqs, int rot_dims, float temp_coef, int temp_every, const int* positions, int n,
-                     hipStream_t stream);
+                     int rot_halves, float rot_mag, float* v_keep, const float* v_first, const float* v_lam, hipStream_t stream);
 int liyab_attention_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
                            const int* block_tables, int max_blocks, const int* tok_seq, const int* tok_pos, int n, float scale,
                            float softcap, int window, const float* bias_table, int max_dist, const float* gate, int64_t gate_stride,
-                           int n_head, int n_kv_head, int dk, int dv, int page_size, int num_pages, hipStream_t stream);
+                           int n_head, int n_kv_head, int dk, int dv, int page_size, int num_pages, const float* sinks, hipStream_t stream);
 
 int liyab_norm_shift(void* out, int out_dtype, float* hbuf, const float* x, const float* w, float offset, float eps, const float* cw, int taps,
                      float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions, const int* seq_starts,
@@ -152,5 +153,13 @@ int liyab_maps_store(const float* src, int64_t ld, const float* cw, int taps, fl
                      int keep_single, hipStream_t stream);
 int liyab_maps_join(void* out, const void* a1, const void* a2, int64_t lda, int dtype, float lam, float eps, float out_scale, int n, int H, int V,
                     int P, hipStream_t stream);
+
+
+int liyab_weighted_sum(float* out, const float* a, const float* b, float wa, float wb, int64_t n, hipStream_t stream);
+int liyab_lru_gates(float* decay, float* input, const float* u, int64_t ldu, const void* wr, const void* wi, int w_dtype, const float* br,
+                    const float* bi, const float* lam, float rate, int n, int blocks, int width, hipStream_t stream);
+int liyab_lru_scan(void* out, int out_dtype, const float* decay, const float* input, const float* y, int64_t ldy, float* state,
+                   int64_t state_stride, int n_slots, const int* seq_starts, const int* positions, const int* state_slots, int n_seqs,
+                   int width, hipStream_t stream);
 
 }  // extern "C"

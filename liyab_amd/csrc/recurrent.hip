@@ -25,7 +25,7 @@
 //   in its row of the output, [n, n_mix * d]), the previous
 //   row taken from the step's rows, from the request's slot, or zero at position 0.
 // liyab_conv_act: out[t, c] = silu(bias[c] + sum_j w[c, j] * in[t - taps + 1 + j, c]) over a request's
-//   own rows in time (the last column of w is the current row's), earlier rows from the ring.
+//   own rows in time (the last column of w is the current row's), earlier rows from the ring; act = 0: without the silu.
 // liyab_gated_group_norm: out = unit_rms_g(y * silu(z)) * w, the root mean square taken over each of
 //   `groups` equal parts of a row.
 #include "common.h"
@@ -475,7 +475,7 @@ __global__ void __launch_bounds__(256)
 conv_act_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ in, int64_t ldi, const float* __restrict__ w,
                 const float* __restrict__ bias, int taps, const float* __restrict__ state, int64_t state_stride, int n_slots,
                 const int* __restrict__ tok_seq, const int* __restrict__ positions, const int* __restrict__ seq_starts,
-                const int* __restrict__ state_slots, int C) {
+                const int* __restrict__ state_slots, int C, int act) {
     const int t = blockIdx.y;
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
@@ -494,7 +494,7 @@ conv_act_kernel(float* __restrict__ out, int64_t ldo, const float* __restrict__ 
         else x = slot_ok ? ring[static_cast<int64_t>(sp % (taps - 1)) * C + c] : 0.0f;
         acc = fmaf(w[static_cast<int64_t>(c) * taps + jt], x, acc);
     }
-    out[static_cast<int64_t>(t) * ldo + c] = silu_f(acc);
+    out[static_cast<int64_t>(t) * ldo + c] = act ? silu_f(acc) : acc;
 }
 
 template <typename T>
@@ -609,7 +609,7 @@ extern "C" int liyab_token_shift(void* out, int dtype, const void* h, const floa
 
 extern "C" int liyab_conv_act(float* out, int64_t ldo, const float* in, int64_t ldi, const float* w, const float* bias, int taps,
                               const float* state, int64_t state_stride, int n_slots, const int* tok_seq, const int* positions,
-                              const int* seq_starts, const int* state_slots, int n, int C, hipStream_t stream) {
+                              const int* seq_starts, const int* state_slots, int n, int C, int act, hipStream_t stream) {
     LIYAB_REQUIRE(out && in && w && tok_seq && positions && seq_starts && state_slots, "conv_act: null pointer");
     LIYAB_REQUIRE(n >= 0 && n <= 65535 && C > 0 && taps >= 1 && ldo >= C && ldi >= C, "conv_act: bad sizes");
     LIYAB_REQUIRE(taps == 1 || (state != nullptr && n_slots > 0 && state_stride >= static_cast<int64_t>(taps - 1) * C),
@@ -617,7 +617,7 @@ extern "C" int liyab_conv_act(float* out, int64_t ldo, const float* in, int64_t 
     if (n == 0) return 0;
     dim3 grid((C + 255) / 256, n);
     conv_act_kernel<<<grid, 256, 0, stream>>>(out, ldo, in, ldi, w, bias, taps, state, state_stride, taps > 1 ? n_slots : 0, tok_seq, positions,
-                                              seq_starts, state_slots, C);
+                                              seq_starts, state_slots, C, act);
     return check_launch("conv_act");
 }
 

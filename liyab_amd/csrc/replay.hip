@@ -23,7 +23,7 @@ namespace liyab {
 namespace replay {
 
 constexpr uint64_t kBlockArg = 0xB10CB10CB10CB10Cull;
-constexpr int kMaxArgs = 32, kMaxBlockWords = 32;
+constexpr int kMaxArgs = 40, kMaxBlockWords = 32;
 
 template <typename T>
 struct Arg {
@@ -121,6 +121,9 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_head_norm_gate),
     LIYAB_ENTRY(liyab_maps_store),
     LIYAB_ENTRY(liyab_maps_join),
+    LIYAB_ENTRY(liyab_weighted_sum),
+    LIYAB_ENTRY(liyab_lru_gates),
+    LIYAB_ENTRY(liyab_lru_scan),
 };
 constexpr int kNumEntries = static_cast<int>(sizeof(kEntries) / sizeof(kEntries[0]));
 

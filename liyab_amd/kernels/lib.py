@@ -79,14 +79,14 @@ _SIGNATURES = {
     "liyab_keep_rows": [P, c_int, c_int, P, P, P, P, P, P, c_int, c_int, P],
     "liyab_latent_store": [P, c_int, P, c_int64, c_int, P, c_float, P, c_int, c_int, c_int, c_int, P],
     "liyab_grouped_product": [P, c_int64, c_int, c_int, P, P, c_int, P, c_int, c_int64, c_int, P, P, c_int, c_int, c_int, P, P, c_int, c_int64,
-                              c_int, c_int, c_int, P],
-    "liyab_moe_route": [P, c_int64, c_int, c_int, c_int, P, P, P],
+                              c_int, c_int, c_int, c_int, c_int, c_int, P],
+    "liyab_moe_route": [P, c_int64, c_int, c_int, c_int, P, P, c_int, c_int, c_int, P],
     "liyab_moe_align": [P, c_int, c_int, c_int, P, P, c_int, P],
-    "liyab_moe_route_align": [P, c_int64, c_int, c_int, c_int, P, P, c_int, P, P, c_int, P],
+    "liyab_moe_route_align": [P, c_int64, c_int, c_int, c_int, P, P, c_int, P, P, c_int, c_int, c_int, c_int, P],
     "liyab_attention_decode_scored": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, P, c_int, c_float, c_int, c_int, c_int,
-                                      c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, c_int, c_float, P, c_int, P],
+                                      c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, c_int, c_float, P, c_int, P, P],
     "liyab_attention_prefill_scored": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
-                                       c_int, c_int, c_int, c_int, c_float, P, c_int, P],
+                                       c_int, c_int, c_int, c_int, c_float, P, c_int, P, P],
     "liyab_gate_rows": [P, c_int, c_int64, P, c_int64, c_int, c_int, P],
     "liyab_dyt": [P, c_int, P, P, P, P, P, c_int, c_int, P],
     "liyab_glu_clamped": [P, c_int, P, c_int64, c_int, c_int, c_float, c_float, c_float, P],
@@ -97,12 +97,12 @@ _SIGNATURES = {
     "liyab_ssd_scan": [P, c_int64, P, c_int64, P, c_int64, P, P, P, P, c_int64, c_int, P, c_int64, c_int, c_int, c_int64, P, P, P, c_int,
                        c_int, c_int, c_int, c_int, c_int, c_int, P, P, P],
     "liyab_token_shift": [P, c_int, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
-    "liyab_conv_act": [P, c_int64, P, c_int64, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, P],
+    "liyab_conv_act": [P, c_int64, P, c_int64, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, c_int, P],
     "liyab_gated_group_norm": [P, c_int, P, c_int64, P, c_int64, P, c_float, c_int, c_int, c_int, P],
     "liyab_qk_prepare": [P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, c_int, P, c_int, c_int, P, P, c_float, P,
-                         c_int, c_float, c_int, P, c_int, P],
+                         c_int, c_float, c_int, P, c_int, c_int, c_float, P, P, P, P],
     "liyab_attention_scored": [P, c_int64, P, c_int64, P, P, c_int, P, c_int, P, P, c_int, c_float, c_float, c_int, P, c_int, P, c_int64,
-                               c_int, c_int, c_int, c_int, c_int, c_int, P],
+                               c_int, c_int, c_int, c_int, c_int, c_int, P, P],
     "liyab_norm_shift": [P, c_int, P, P, P, c_float, c_float, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, c_int, c_int, P],
     "liyab_ring_keep": [P, c_int64, c_int, c_int, P, c_int64, c_int, P, P, P, P, P, c_int, P],
     "liyab_normed_powers": [P, c_int, P, c_int64, c_int, c_int, P, c_float, P],
@@ -115,6 +115,9 @@ _SIGNATURES = {
     "liyab_maps_store": [P, c_int64, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, P, c_int, c_int, P, P, P, P, c_int, c_int, c_int,
                          c_int, c_int, c_int, c_int, P],
     "liyab_maps_join": [P, P, P, c_int64, c_int, c_float, c_float, c_float, c_int, c_int, c_int, c_int, P],
+    "liyab_weighted_sum": [P, P, P, c_float, c_float, c_int64, P],
+    "liyab_lru_gates": [P, P, P, c_int64, P, P, c_int, P, P, P, c_float, c_int, c_int, c_int, P],
+    "liyab_lru_scan": [P, c_int, P, P, P, c_int64, P, c_int64, c_int, P, P, P, c_int, c_int, P],
 }
 
 

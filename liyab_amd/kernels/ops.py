@@ -782,7 +782,8 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
                      scale: float, window: int = 0, n_splits: int = 1, partials: Optional[torch.Tensor] = None,
                      tok_list: Optional[torch.Tensor] = None, n_tokens: Optional[int] = None, waves: int = 4,
                      rows_are_requests: bool = False, leave_splits: bool = False, chunk: int = 0,
-                     num_pages: Optional[int] = None, softcap: float = 0.0, bias_table: Optional[torch.Tensor] = None) -> None:
+                     num_pages: Optional[int] = None, softcap: float = 0.0, bias_table: Optional[torch.Tensor] = None,
+                     sinks: Optional[torch.Tensor] = None) -> None:
     """Each token on its own over its request's cache (bfloat16, or float32 throughout), its keys cut into `n_splits`.
     With `tok_list` (int32) only those rows are computed. `rows_are_requests`: row t belongs to
     request t (every request brings one token), which saves the kernel a lookup. With
@@ -791,7 +792,8 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
     that merges them (`gemm_att_parts`). `chunk` > 0: split z takes keys [z * chunk, (z + 1) * chunk) of a
     token's keys instead of an equal share (`n_splits * chunk` must cover the longest context): a token's
     sums then follow from its position alone. `softcap` > 0: scores become cap * tanh(score / cap); `bias_table` (float32
-    [distances, heads]): + table[min(position - key, distances - 1), head]."""
+    [distances, heads]): + table[min(position - key, distances - 1), head]; `sinks` (float32 [heads]): exp(sinks[head]) joins
+    the softmax's denominator (a learned logit with no key and no value)."""
     if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise KernelError("attention: caches must be contiguous [pages, kv_heads, page_size, head_dim] of one shape")
     _, hkv, page, hd = k_cache.shape
@@ -821,8 +823,11 @@ def attention_decode(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
             dtype_code(q.dtype), block_tables.data_ptr(), block_tables.shape[1], _ptr(tok_list), tok_seq.data_ptr(), tok_pos.data_ptr(),
             n, float(scale), int(window), n_head, hkv, hd, page, n_splits, int(chunk), waves, 1 if rows_are_requests else 0,
             _ptr(partials), 1 if leave_splits else 0, _pages(k_cache, num_pages))
-    if softcap > 0 or bias_table is not None:
-        _lib.call("liyab_attention_decode_scored", *args, float(softcap), _ptr(bias_table), _bias_rows(bias_table, n_head) - 1, _stream())
+    _f32vec(sinks, "sinks", n_head)
+    if softcap > 0 or bias_table is not None or sinks is not None:
+        if sinks is not None and leave_splits:
+            raise KernelError("attention_decode: splits left unmerged take no sink")
+        _lib.call("liyab_attention_decode_scored", *args, float(softcap), _ptr(bias_table), _bias_rows(bias_table, n_head) - 1, _ptr(sinks), _stream())
     else:
         _lib.call("liyab_attention_decode", *args, _stream())
 
@@ -853,7 +858,7 @@ def attention_merge(out: torch.Tensor, partials: torch.Tensor) -> None:
 def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, work: torch.Tensor, n_tiles: int, *, n_head: int, scale: float,
                       window: int = 0, tile: int = 128, ksplit: int = 1, num_pages: Optional[int] = None, softcap: float = 0.0,
-                      bias_table: Optional[torch.Tensor] = None) -> None:
+                      bias_table: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None) -> None:
     """Tiles of up to `tile` (64 or 128) consecutive queries of one request over its bfloat16
     cache, on the matrix cores; `ksplit` waves (1, 2, or 4 with tiles of 64) share the keys of
     32 queries. work: int32 [n_tiles, 4] = (request index, first row, first
@@ -875,8 +880,9 @@ def attention_prefill(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     args = (out.data_ptr(), os_, q.data_ptr(), qs, k_cache.data_ptr(), v_cache.data_ptr(),
             block_tables.data_ptr(), block_tables.shape[1], work.data_ptr(), n_tiles, int(tile), int(ksplit), float(scale), int(window),
             n_head, hkv, hd, page, _pages(k_cache, num_pages))
-    if softcap > 0 or bias_table is not None:  # (see attention_decode)
-        _lib.call("liyab_attention_prefill_scored", *args, float(softcap), _ptr(bias_table), _bias_rows(bias_table, n_head) - 1, _stream())
+    _f32vec(sinks, "sinks", n_head)
+    if softcap > 0 or bias_table is not None or sinks is not None:  # (see attention_decode)
+        _lib.call("liyab_attention_prefill_scored", *args, float(softcap), _ptr(bias_table), _bias_rows(bias_table, n_head) - 1, _ptr(sinks), _stream())
     else:
         _lib.call("liyab_attention_prefill", *args, _stream())
 
@@ -962,17 +968,20 @@ def attention_takes(head_dim: int) -> bool:
 
 def attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
               block_tables: torch.Tensor, ctx, *, n_head: int, scale: float, window: int = 0,
-              splits_ok: bool = False, softcap: float = 0.0, bias_table: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+              splits_ok: bool = False, softcap: float = 0.0, bias_table: Optional[torch.Tensor] = None,
+              sinks: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
     """Attention of the step's tokens over their requests' cached keys and values; the kernel
     is chosen from the step's shape (`ctx` is the step's StepContext; `ctx.plans["attention"]`
     says how the step's tokens are cut, see parts/attention.py; without it every token goes to
     the plain kernel). With `splits_ok`, a step of few tokens may leave `out` unwritten and
     return the splits of each (token, head) pair instead, float32 [tokens, heads, splits, head
-    size + 4], for `gemm_att_parts`. `softcap`, `bias_table`: what is done to the scores before the softmax (see
-    `attention_decode`); every kernel below does the same."""
+    size + 4], for `gemm_att_parts`. `softcap`, `bias_table`: what is done to the scores before the softmax, `sinks`: a learned
+    logit a head in its denominator (see `attention_decode`); every kernel below does the same."""
     hd = k_cache.shape[3]
     host = ctx.host
-    scored = dict(softcap=softcap, bias_table=bias_table) if softcap > 0 or bias_table is not None else {}
+    scored = dict(softcap=softcap, bias_table=bias_table, sinks=sinks) if softcap > 0 or bias_table is not None or sinks is not None else {}
+    if sinks is not None and splits_ok:
+        raise KernelError("attention: splits left to the caller take no sink")
     plan = ctx.plans.get("attention")
     fast = (plan is not None and q.dtype == torch.bfloat16 and hd % 8 == 0 and q.stride(0) % 8 == 0
             and out.stride(0) % 8 == 0)
@@ -1204,7 +1213,7 @@ def heads_product(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, gate: Opt
                             and w.data_ptr() % 16 == 0) else GROUPED_ROWS
     _lib.call("liyab_grouped_product", a.data_ptr(), lda, 1, K, w.data_ptr(), None, dtype_code(a.dtype), out.data_ptr(),
               dtype_code(out.dtype), ldo, N, None, None, (n + block - 1) // block, block, H, None, _ptr(gate),
-              dtype_code(gate.dtype) if gate is not None else F32, gs, n, N, K, _stream())
+              dtype_code(gate.dtype) if gate is not None else F32, gs, n, N, K, 0, 1, 0, _stream())
 
 
 MOE_MAX_TOP = 64
@@ -1226,12 +1235,17 @@ def moe_block(n_entries: int, n_experts: int, dtype: torch.dtype, *inner_sizes: 
     return SKINNY_ROWS if few else GROUPED_ROWS
 
 
+MOE_MAX_GROUPS = 64
+
+
 def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, rows_list: torch.Tensor,
-              tile_group: torch.Tensor, block: int = GROUPED_ROWS) -> None:
+              tile_group: torch.Tensor, block: int = GROUPED_ROWS, groups: Optional[tuple] = None) -> None:
     """From float32 router logits [n, experts] (rows may be strided): ids int32 and weights float32 [n,
     top] (the experts with the largest logits, softmax over those alone), and the entries t * top + k
     listed by expert in tiles of `block` places: rows_list int32 [tiles * block] (-1: empty), tile_group
-    int32 [tiles] (-1: unused), tiles = moe_tiles(n * top, experts, block)."""
+    int32 [tiles] (-1: unused), tiles = moe_tiles(n * top, experts, block). `groups` = (count, keep): the choice among groups
+    of experts instead: softmax over all experts, the experts in `count` equal groups of neighbours, only those of the `keep`
+    groups with the largest member can be chosen, the weights the chosen scores divided by their sum."""
     ld = _rows(logits, "logits")
     n, E = logits.shape
     if logits.dtype != torch.float32:
@@ -1247,20 +1261,27 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
     _dev(weights, "weights")
     if weights.dtype != torch.float32 or weights.numel() < n * top or not weights.is_contiguous():
         raise KernelError("moe_route: weights must be contiguous float32 [n, top]")
+    mode, count, keep = 0, 1, 1
+    if groups is not None:
+        mode, count, keep = 1, int(groups[0]), int(groups[1])
+        if not (1 <= count <= MOE_MAX_GROUPS and E % count == 0 and 1 <= keep <= count and top <= keep * (E // count)):
+            raise KernelError(f"moe_route: {keep} of {count} groups of {E} experts do not hold {top} choices (at most {MOE_MAX_GROUPS} groups)")
     if n <= 1024:  # one launch: a thread routes a token, then the workgroup lists the entries
         _lib.call("liyab_moe_route_align", logits.data_ptr(), ld, n, E, top, ids.data_ptr(), weights.data_ptr(), block,
-                  rows_list.data_ptr(), tile_group.data_ptr(), tiles, _stream())
+                  rows_list.data_ptr(), tile_group.data_ptr(), tiles, mode, count, keep, _stream())
         return
-    _lib.call("liyab_moe_route", logits.data_ptr(), ld, n, E, top, ids.data_ptr(), weights.data_ptr(), _stream())
+    _lib.call("liyab_moe_route", logits.data_ptr(), ld, n, E, top, ids.data_ptr(), weights.data_ptr(), mode, count, keep, _stream())
     _lib.call("liyab_moe_align", ids.data_ptr(), n * top, E, block, rows_list.data_ptr(), tile_group.data_ptr(), tiles, _stream())
 
 
 def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Optional[torch.Tensor], rows_list: torch.Tensor,
-                tile_group: torch.Tensor, *, a_div: int = 1, row_scale: Optional[torch.Tensor] = None, block: int = GROUPED_ROWS) -> None:
+                tile_group: torch.Tensor, *, a_div: int = 1, row_scale: Optional[torch.Tensor] = None, block: int = GROUPED_ROWS,
+                act: str = "none", out_div: int = 1, out_extra: int = 0) -> None:
     """For every listed entry e of expert g: out[e] = f(a[e // a_div] . w0[g]^T, a[e // a_div] . w1[g]^T) *
     row_scale[e], f(u, v) = silu(u) * v with two matrices and u with one. a [*, K] and out [entries, N]
     contiguous, w0 / w1 [experts, N, K] in a's dtype; rows_list and tile_group as `moe_route` leaves them for
-    tiles of `block` places."""
+    tiles of `block` places. `act` = "relu2" (one matrix): f(u) = relu(u)^2. `out_extra`: rows of `out` left free behind each
+    `out_div` rows (a token's entries), which another product fills: entry e then lies at row e + (e // out_div) * out_extra."""
     _dev(w0, "w0")
     if w0.dim() != 3 or not w0.is_contiguous() or w0.dtype != a.dtype:
         raise KernelError(f"moe_product: w0 must be contiguous [experts, N, K] in a's dtype, got {tuple(w0.shape)} {w0.dtype}")
@@ -1268,7 +1289,9 @@ def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Option
     if w1 is not None and (tuple(w1.shape) != (E, N, K) or not w1.is_contiguous() or w1.dtype != a.dtype):
         raise KernelError("moe_product: w1 must match w0")
     lda, ldo = _rows(a, "a"), _rows(out, "out")
-    entries = out.shape[0]
+    if act not in ("none", "relu2") or (act != "none" and w1 is not None) or out_extra < 0 or out_div < 1 or (out_extra and out.shape[0] % (out_div + out_extra)):
+        raise KernelError(f"moe_product: activation '{act}' / {out_extra} free rows a token are not taken here")
+    entries = out.shape[0] // (out_div + out_extra) * out_div if out_extra else out.shape[0]
     if a.shape[1] != K or out.shape[1] != N or a_div < 1 or a.shape[0] * a_div < entries:
         raise KernelError(f"moe_product: a {tuple(a.shape)} / out {tuple(out.shape)} do not fit [{E}, {N}, {K}] with {a_div} entries a row")
     tiles = tile_group.numel()
@@ -1284,7 +1307,7 @@ def moe_product(out: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, w1: Option
             raise KernelError("moe_product: row_scale must be contiguous float32 [entries]")
     _lib.call("liyab_grouped_product", a.data_ptr(), lda, a_div, 0, w0.data_ptr(), _ptr(w1), dtype_code(a.dtype), out.data_ptr(),
               dtype_code(out.dtype), ldo, 0, rows_list.data_ptr(), tile_group.data_ptr(), tiles, block, E, _ptr(row_scale), None, F32, 0,
-              entries, N, K, _stream())
+              entries, N, K, 1 if act == "relu2" else 0, int(out_div), int(out_extra), _stream())
 
 
 # -- norms without statistics, clamped gated activations, two sublayers' results joined ------------
@@ -1318,7 +1341,7 @@ def glu_clamped(out: torch.Tensor, gu: torch.Tensor, limit: float, slope: float,
     _lib.call("liyab_glu_clamped", out.data_ptr(), dtype_code(out.dtype), gu.data_ptr(), ld, n, ff, float(limit), float(slope), float(shift), _stream())
 
 
-ACTIVATE = {"tanh": 0, "silu": 1, "sigmoid": 2}
+ACTIVATE = {"tanh": 0, "silu": 1, "sigmoid": 2, "relu2": 3}
 
 
 def activate(out: torch.Tensor, x: torch.Tensor, op: str) -> None:
@@ -1436,8 +1459,8 @@ def wkv_scan(out: torch.Tensor, proj: torch.Tensor, w0: torch.Tensor, u: torch.T
 
 
 def conv_act(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
-             ring_off: int, ctx) -> None:
-    """out[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - taps + 1 + j, c]) over each request's own rows in time; x, out float32
+             ring_off: int, ctx, act: bool = True) -> None:
+    """(`act` False: without the silu.) out[t, c] = silu(bias[c] + sum_j weight[c, j] * x[t - taps + 1 + j, c]) over each request's own rows in time; x, out float32
     rows (columns of wider rows are fine), weight float32 [C, taps]; the rows before a request's first row of the step come from
     state[slot, ring_off + (position % (taps - 1)) * C + c], zeros before position 0."""
     ldo, ldi = _rows(out, "out"), _rows(x, "x")
@@ -1457,7 +1480,8 @@ def conv_act(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Opt
         slots, base = state.shape[0], state.data_ptr() + 4 * ring_off
     _step_lists(ctx, n)
     _lib.call("liyab_conv_act", out.data_ptr(), ldo, x.data_ptr(), ldi, weight.data_ptr(), _ptr(bias), taps, base, stride, slots,
-              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, C, _stream())
+              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, C, 1 if act else 0,
+              _stream())
 
 
 def ssd_scan(y: torch.Tensor, xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
@@ -1515,13 +1539,18 @@ def gated_group_norm(out: torch.Tensor, y: torch.Tensor, z: torch.Tensor, weight
 def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slots: torch.Tensor, positions: torch.Tensor,
                *, q_off: int, k_off: int, v_off: int, n_head: int, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
                eps: float = 0.0, freqs: Optional[torch.Tensor] = None, rot_dims: int = 0, temp_coef: float = 0.0, temp_every: int = 0,
-               num_pages: Optional[int] = None, head_dim: Optional[int] = None, value_dim: Optional[int] = None) -> None:
+               num_pages: Optional[int] = None, head_dim: Optional[int] = None, value_dim: Optional[int] = None, rot_halves: bool = False,
+               rot_mag: float = 1.0, v_keep: Optional[torch.Tensor] = None, v_first: Optional[torch.Tensor] = None,
+               v_lam: Optional[torch.Tensor] = None) -> None:
     """From a projection's float32 rows `src` (queries at column q_off, keys at k_off, values at v_off, which may be k_off) to
     queries in `q_out` [n, heads * dk] and keys and values in their slots of the pages (k_cache [pages, kv_heads, page, dk],
     v_cache [.., dv]), all in the compute dtype. Per head, each optional: a root-mean-square norm with a weight [dk] (queries,
     keys), pairs (2i, 2i + 1) of the first rot_dims entries turned by position * freqs[i] (queries, keys), the query times
     1 + temp_coef * ln(floor((position + 1) / temp_every) + 1). A slot outside the pages is not written. `head_dim`,
-    `value_dim`: the heads' own widths where the caches' rows (and the queries') are wider, zeros behind the heads."""
+    `value_dim`: the heads' own widths where the caches' rows (and the queries') are wider, zeros behind the heads. `rot_halves`:
+    the turned pairs are (i, i + rot_dims / 2) instead; `rot_mag` multiplies cosine and sine. `v_keep` (float32 [n, kv_heads * dv]) gets
+    the values as projected, for later layers of the step; `v_first` (such rows) and `v_lam` (one float32 on the device): the values
+    cached are (1 - lam) v + lam v_first."""
     ld = _rows(src, "src")
     n = src.shape[0]
     _dev(q_out, "q_out")
@@ -1546,17 +1575,24 @@ def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_
         _f32vec(freqs, "freqs", rot_dims // 2)
     _i32(slots, "slots", n)
     _i32(positions, "positions", n)
+    for kept, what in ((v_keep, "v_keep"), (v_first, "v_first")):
+        _f32vec(kept, what, n * G * dv)
+    _f32vec(v_lam, "v_lam", 1)
+    if (v_first is None) != (v_lam is None) or (v_keep is not None and v_first is not None):
+        raise KernelError("qk_prepare: values are kept, or mixed with kept ones at a rate")
     _lib.call("liyab_qk_prepare", src.data_ptr(), ld, q_off, k_off, v_off, n_head, G, dk, dv, dk_out, dv_out, q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
               dtype_code(q_out.dtype), slots.data_ptr(), page, _pages(k_cache, num_pages), _ptr(q_norm), _ptr(k_norm), float(eps),
-              _ptr(freqs) if rot_dims else None, rot_dims, float(temp_coef), int(temp_every), positions.data_ptr(), n, _stream())
+              _ptr(freqs) if rot_dims else None, rot_dims, float(temp_coef), int(temp_every), positions.data_ptr(), n,
+              1 if rot_halves else 0, float(rot_mag), _ptr(v_keep), _ptr(v_first), _ptr(v_lam), _stream())
 
 
 def attention_scored(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor, ctx, *,
                      n_head: int, scale: float, softcap: float = 0.0, window: int = 0, bias_table: Optional[torch.Tensor] = None,
-                     gate: Optional[torch.Tensor] = None, num_pages: Optional[int] = None) -> None:
+                     gate: Optional[torch.Tensor] = None, num_pages: Optional[int] = None, sinks: Optional[torch.Tensor] = None) -> None:
     """Causal attention of the step's rows over their requests' pages with score = scale * q . k, then cap * tanh(score / cap)
     (softcap > 0), then + bias_table[min(distance, rows - 1), head] (float32 [rows, heads]); softmax in 32-bit; values `dv` wide.
-    out [n, heads * dv] = result * sigmoid(gate) (gate: float32 rows [n, heads * dv], or None)."""
+    out [n, heads * dv] = result * sigmoid(gate) (gate: float32 rows [n, heads * dv], or None). `sinks` (float32 [heads]):
+    exp(sinks[head]) joins the softmax's denominator."""
     _dev(out, "out")
     _dev(q, "q")
     n = out.shape[0]
@@ -1585,9 +1621,10 @@ def attention_scored(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
         gs = _rows(gate, "gate")
         if gate.dtype != torch.float32 or tuple(gate.shape) != (n, n_head * dv):
             raise KernelError("attention_scored: the gate must be float32 rows [n, heads * dv]")
+    _f32vec(sinks, "sinks", n_head)
     _lib.call("liyab_attention_scored", out.data_ptr(), so, q.data_ptr(), sq, k_cache.data_ptr(), v_cache.data_ptr(), dtype_code(q.dtype),
               block_tables.data_ptr(), block_tables.shape[1], ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), n, float(scale), float(softcap),
-              int(window), _ptr(bias_table), max_dist, _ptr(gate), gs, n_head, G, dk, dv, page, _pages(k_cache, num_pages), _stream())
+              int(window), _ptr(bias_table), max_dist, _ptr(gate), gs, n_head, G, dk, dv, page, _pages(k_cache, num_pages), _ptr(sinks), _stream())
 
 
 def gate_rows(x: torch.Tensor, gate: torch.Tensor) -> None:
@@ -1826,3 +1863,56 @@ def maps_join(out: torch.Tensor, a1: torch.Tensor, a2: torch.Tensor, lam: float,
         raise KernelError(f"maps_join: out must be contiguous [{n}, {H * V}]")
     _lib.call("liyab_maps_join", out.data_ptr(), a1.data_ptr(), a2.data_ptr(), lda, dtype_code(out.dtype), float(lam), float(eps), float(out_scale),
               n, H, V, P, _stream())
+
+
+# -- a linear recurrence a channel with real gates; two results joined with constant weights ---------------------
+def weighted_sum(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, wa: float, wb: float) -> None:
+    """out = wa * a + wb * b; contiguous float32 tensors of one shape (out may be a or b)."""
+    for t, what in ((out, "out"), (a, "a"), (b, "b")):
+        _dev(t, what)
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.shape != out.shape:
+            raise KernelError("weighted_sum: out, a and b must be contiguous float32 of one shape")
+    _lib.call("liyab_weighted_sum", out.data_ptr(), a.data_ptr(), b.data_ptr(), float(wa), float(wb), out.numel(), _stream())
+
+
+def lru_gates(decay: torch.Tensor, gated: torch.Tensor, u: torch.Tensor, wr: torch.Tensor, wi: torch.Tensor, br: torch.Tensor, bi: torch.Tensor,
+              lam: torch.Tensor, rate: float) -> None:
+    """From the recurrence's input u (float32 rows [n, width], columns of wider rows are fine) in `blocks` equal parts: r = sigmoid(Wr[b]
+    u_b + br), i = sigmoid(Wi[b] u_b + bi), decay = exp(-rate * r * softplus(lam)), gated = sqrt(1 - decay^2) * i * u; decay and gated
+    contiguous float32 [n, width]. wr, wi [blocks, in, out] (a part's matrix transposed), bfloat16 or float32; br, bi, lam float32 [width]."""
+    ldu = _rows(u, "u")
+    n, W = u.shape
+    _dev(wr, "wr")
+    if wr.dim() != 3 or wr.shape[1] != wr.shape[2] or wr.shape[0] * wr.shape[1] != W or wr.shape != wi.shape or wr.dtype != wi.dtype \
+            or not wr.is_contiguous() or not wi.is_contiguous():
+        raise KernelError(f"lru_gates: the gates' matrices must be contiguous [blocks, in, out] over {W} channels, got {tuple(wr.shape)} / {tuple(wi.shape)}")
+    if u.dtype != torch.float32:
+        raise KernelError("lru_gates: u must be float32")
+    for t, what in ((decay, "decay"), (gated, "gated")):
+        _dev(t, what)
+        if t.dtype != torch.float32 or tuple(t.shape) != (n, W) or not t.is_contiguous():
+            raise KernelError(f"lru_gates: {what} must be contiguous float32 [{n}, {W}]")
+    _f32vec(br, "br", W)
+    _f32vec(bi, "bi", W)
+    _f32vec(lam, "lam", W)
+    _lib.call("liyab_lru_gates", decay.data_ptr(), gated.data_ptr(), u.data_ptr(), ldu, wr.data_ptr(), wi.data_ptr(), dtype_code(wr.dtype), br.data_ptr(),
+              bi.data_ptr(), lam.data_ptr(), float(rate), n, wr.shape[0], W, _stream())
+
+
+def lru_scan(out: torch.Tensor, decay: torch.Tensor, gated: torch.Tensor, y: torch.Tensor, state: torch.Tensor, ctx) -> None:
+    """S_t = decay_t * S_(t-1) + gated_t along each request's rows of the step, from state[slot, :width] (zero at position 0), which gets
+    the last S; out[t] = S_t * gelu_tanh(y_t) in out's dtype. decay, gated float32 [n, width]; y float32 rows (columns of wider rows are
+    fine); out contiguous [n, width]."""
+    ldy = _rows(y, "y")
+    n, W = y.shape
+    stride = _state(state, "lru_scan")
+    _dev(out, "out")
+    if y.dtype != torch.float32 or tuple(out.shape) != (n, W) or not out.is_contiguous() or ctx.n_tokens != n or stride < W:
+        raise KernelError("lru_scan: y must be the step's float32 rows, out contiguous of the same shape, and the slot must hold a row")
+    for t, what in ((decay, "decay"), (gated, "gated")):
+        _dev(t, what)
+        if t.dtype != torch.float32 or tuple(t.shape) != (n, W) or not t.is_contiguous():
+            raise KernelError(f"lru_scan: {what} must be contiguous float32 [{n}, {W}]")
+    _step_lists(ctx, n)
+    _lib.call("liyab_lru_scan", out.data_ptr(), dtype_code(out.dtype), decay.data_ptr(), gated.data_ptr(), y.data_ptr(), ldy, state.data_ptr(), stride,
+              state.shape[0], ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, W, _stream())

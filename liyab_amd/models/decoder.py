@@ -129,7 +129,8 @@ class DecoderModel:
             # what a block may have of its own between the stream and its sublayers (a convolution on a
             # sublayer's input, gates on the results): built here, handed over by name where the plan has them
             extras = {}
-            for name, family in (("input_conv", "conv"), ("ffn_conv", "conv"), ("gate_mixer", "gate"), ("gate_ffn", "gate")):
+            for name, family in (("input_conv", "conv"), ("ffn_conv", "conv"), ("gate_mixer", "gate"), ("gate_ffn", "gate"),
+                                 ("post_norm_mixer", "norm"), ("post_norm_ffn", "norm")):
                 extra = getattr(spec, name, None)
                 if extra is not None:
                     extras[name] = build_part(family, extra, store, dtype)
@@ -166,7 +167,7 @@ class DecoderModel:
         # the head see the wanted rows only.
         every = [self.embedding, self.residual_position] + list(self.entries.values())
         for block in self.blocks:
-            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn", "conv", "ffn_conv", "gate_mixer", "gate_ffn")]
+            every += [block] + [getattr(block, a, None) for a in ("mixer", "ffn", "norm_mixer", "norm_ffn", "conv", "ffn_conv", "gate_mixer", "gate_ffn", "post_norm_mixer", "post_norm_ffn")]
         self.takes_padding_rows = all(bool(getattr(part, "takes_padding_rows", False)) for part in every if part is not None)
 
     # -- what the cache manager needs to know ---------------------------------

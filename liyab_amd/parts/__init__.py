@@ -16,5 +16,5 @@ from .registry import (  # noqa: F401
     register_position,
 )
 from .norms import Normed, as_tensor  # noqa: F401
-from . import (attention, block, conv, delta_rule, differential_attention, embeddings, feedforward, head, latent_attention, norms, recurrent, reentry,  # noqa: F401
+from . import (attention, block, conv, delta_rule, differential_attention, embeddings, feedforward, gated_recurrence, head, latent_attention, norms, recurrent, reentry,  # noqa: F401
                routed, scored_attention, side_by_side)  # noqa: F401  (register themselves)

@@ -205,6 +205,52 @@ class PostNormGatedBlock:
 register_block("post_norm_gated", PostNormGatedBlock)
 
 
+class SandwichBlock:
+    """x += post_norm_mixer(mixer(norm_mixer(x))); x += post_norm_ffn(ffn(norm_ffn(x))): a norm before each sublayer and a
+    root-mean-square norm behind it. The sublayers leave their 32-bit results to the block (`forward(..., out=)`; a
+    feed-forward may leave several rows a token, `rows_a_token`), and one kernel a sublayer takes the sum of a token's rows, its
+    root mean square, the weight and the addition into the 32-bit stream. The feed-forward is optional."""
+
+    replayable = True
+    takes_padding_rows = True
+    takes_pending = False
+
+    def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn, post_norm_mixer=None, post_norm_ffn=None):
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn if ffn is not None else None
+        self.post_norm_mixer, self.post_norm_ffn = post_norm_mixer, post_norm_ffn if ffn is not None else None
+        self.mixer_phase = getattr(getattr(spec, "mixer", None), "kind", "mixer")
+        self.ffn_phase = getattr(getattr(spec, "ffn", None), "kind", "ffn")
+        for part, what in ((mixer, "mixer"), (ffn, "feed-forward")):
+            if part is not None and "out" not in part.forward.__code__.co_varnames:
+                raise ValueError(f"a sandwich block needs a {what} that can leave its result to the block (forward(..., out=))")
+        for norm in (post_norm_mixer, post_norm_ffn if ffn is not None else post_norm_mixer):
+            if norm is None or not getattr(norm, "root_mean_square", False):
+                raise ValueError("a sandwich block's row update applies a root-mean-square norm behind each sublayer (kind 'rmsnorm')")
+        if norm_mixer is None or (ffn is not None and norm_ffn is None):
+            raise ValueError("a sandwich block has a norm before each sublayer")
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache, state, writes_cache: bool = True):
+        ws, n, d = ctx.workspace, x.shape[0], x.shape[1]
+        if ctx.phases is not None:
+            ctx.phases.mark(self.mixer_phase)
+        h = self.norm_mixer.forward(x, ctx, name="block_in")
+        y = ws.get("sublayer_out", (n, d), torch.float32)
+        self.mixer.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=y)
+        ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps)
+        if self.ffn is not None:
+            if ctx.phases is not None:
+                ctx.phases.mark(self.ffn_phase)
+            h = self.norm_ffn.forward(x, ctx, name="block_in")
+            k = int(getattr(self.ffn, "rows_a_token", 1))
+            y = ws.get("sublayer_rows", (n * k, d), torch.float32) if k > 1 else y
+            self.ffn.forward(h, ctx, None, out=y)
+            ops.gated_norm_add(x, y, self.post_norm_ffn.weight, self.post_norm_ffn.eps, n_sum=k)
+        return None
+
+
+register_block("sandwich", SandwichBlock)
+
+
 class ParallelPairBlock:
     """x += mixer(c1(norm_mixer(x))) + ffn(c2(norm_ffn(x))): two root-mean-square norms of the same stream (they share the root
     mean square, so one pass over a row gives both), each followed by a short causal convolution over time of its own, h <- h +

@@ -22,7 +22,8 @@ from .registry import register_mixer
 def rotary_frequencies(rot) -> np.ndarray:
     """f_i = base^(-2i / dims) for i < dims / 2, the long wavelengths stretched as `rot.scaling` = (factor, low, high,
     original) says: with wavelength l = 2 pi / f, f stays for l < original / high, becomes f / factor for l > original /
-    low, and in between is (1 - s) f / factor + s f with s = (original / l - low) / (high - low). float64."""
+    low, and in between is (1 - s) f / factor + s f with s = (original / l - low) / (high - low); or as `rot.ramp` = (factor,
+    fast, slow, original) says, by the entry's number (see RotarySpec). float64."""
     f = np.array([float(rot.base) ** (-2.0 * i / rot.dims) for i in range(rot.dims // 2)], dtype=np.float64)
     if rot.scaling is not None:
         factor, low, high, original = (float(v) for v in rot.scaling)
@@ -35,7 +36,25 @@ def rotary_frequencies(rot) -> np.ndarray:
             else:
                 s = (original / wavelength - low) / (high - low)
                 f[i] = (1.0 - s) * fi / factor + s * fi
+    if getattr(rot, "ramp", None) is not None:
+        factor, fast, slow, original = (float(v) for v in rot.ramp)
+
+        def at(turns: float) -> float:
+            return rot.dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(rot.base)))
+
+        lo = max(math.floor(at(fast)), 0)
+        hi = min(math.ceil(at(slow)), rot.dims - 1)
+        for i, fi in enumerate(f):
+            r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            f[i] = fi / factor * r + fi * (1.0 - r)
     return f
+
+
+def rotary_magnitude(rot) -> float:
+    """What cosine and sine are multiplied by: 1, or ramp_magnitude * ln(factor) + 1 with a ramp."""
+    if getattr(rot, "ramp", None) is None:
+        return 1.0
+    return float(rot.ramp_magnitude) * math.log(float(rot.ramp[0])) + 1.0
 
 
 def distance_rows(n_rows: int, far: int) -> np.ndarray:
@@ -92,6 +111,22 @@ class ScoredAttention:
             shapes.append((H * V, d))
             at += H * V
         self.in_weight = store.fetch_joined(srcs, shapes, "matrix", "rows")
+        # biases on the projections of queries, keys and values: one vector over the joint product's columns, zeros for the gate's
+        self.in_bias = None
+        if getattr(spec, "biased", False):
+            names = [t["q_bias"], t["k_bias"]] + ([] if self.values_are_keys else [t["v_bias"]])
+            bias = store.fetch_joined(names, [(r[0],) for r in shapes[:len(names)]], "vector", "rows")
+            if self.gated:
+                bias = store.derived(("bias_zeros_behind", tuple(b.name for b in names), H * V),
+                                     lambda: torch.cat([bias, torch.zeros(H * V, dtype=torch.float32, device=bias.device)]).contiguous())
+            self.in_bias = bias
+        self.sinks = store.fetch(t["sink"], (H,), "vector") if getattr(spec, "sink", False) else None
+        # values shared between layers of a step: the first such layer keeps its values as projected, the later ones mix theirs
+        # with those at a learned rate (one float, read on the device); both find the rows under one name in the step's workspace
+        self.value_mix = getattr(spec, "value_mix", "") or ""
+        if self.value_mix not in ("", "first", "later") or (self.value_mix and self.values_are_keys):
+            raise ValueError(f"scored attention: value_mix '{self.value_mix}'")
+        self.v_lam = store.fetch(t["vmix"], (), "vector").reshape(1) if self.value_mix else None
         self.out_weight = store.fetch(t["out"], (d, H * V), "matrix")
         # Keys and values of different widths: both planes of the pages as wide as the wider (a multiple of 8), zeros behind the
         # narrower heads, which is what the engine's paged attention kernels take; zeros in keys and queries add nothing to a
@@ -103,13 +138,14 @@ class ScoredAttention:
             self.out_weight = store.derived(("padded_heads", t["out"].name, P), lambda: torch.nn.functional.pad(w.view(d, H, V), (0, P - V)).reshape(d, H * P).contiguous())
         self.q_norm = store.fetch(t["q_norm"], (D,), "vector") if spec.qk_norm else None
         self.k_norm = store.fetch(t["k_norm"], (D,), "vector") if spec.qk_norm else None
-        self.rot_dims, self.freqs = 0, None
+        self.rot_dims, self.freqs, self.rot_halves, self.rot_mag = 0, None, False, 1.0
         if spec.rotary is not None:
             rot = spec.rotary
             if rot.dims % 2 or not 0 < rot.dims <= D:
                 raise ValueError(f"rotary encoding over {rot.dims} of {D} entries")
             self.rot_dims = int(rot.dims)
-            self.freqs = store.derived(("rotary", rot.dims, rot.base, rot.scaling),
+            self.rot_halves, self.rot_mag = bool(getattr(rot, "halves", False)), rotary_magnitude(rot)
+            self.freqs = store.derived(("rotary", rot.dims, rot.base, rot.scaling, getattr(rot, "ramp", None)),
                                        lambda: torch.from_numpy(rotary_frequencies(rot).astype(np.float32)).to(self.out_weight.device))
         self.temp_coef, self.temp_every = (float(spec.q_temp[0]), int(spec.q_temp[1])) if spec.q_temp else (0.0, 0)
         self.bias_table = None
@@ -121,6 +157,12 @@ class ScoredAttention:
             self.bias_table = store.derived(("distance_bias", t["rel"].name, far),
                                             lambda: rel[torch.from_numpy(distance_rows(rows, far)).to(rel.device)].contiguous())
 
+    def _shared_values(self, ws, n: int) -> dict:
+        if not self.value_mix:
+            return {}
+        rows = ws.get("first_values", (n * self.n_kv_head * self.value_dim,), torch.float32)
+        return {"v_keep": rows} if self.value_mix == "first" else {"v_first": rows, "v_lam": self.v_lam}
+
     def cache_spec(self) -> Optional[KVSpec]:
         return KVSpec(self.n_kv_head, self.head_dim, self.window,
                       rows=(("k", self.n_kv_head, self.row_dim or self.head_dim), ("v", self.n_kv_head, self.row_dim or self.value_dim)))
@@ -131,32 +173,33 @@ class ScoredAttention:
     def forward(self, h, ctx: StepContext, cache: LayerCache, state, residual: Optional[torch.Tensor],
                 writes_cache: bool = True, out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None):
         """Adds the mixer's result into `residual`, or, with `out` (float32 [n, width]), leaves it there. `proj`: the input
-        projection's 32-bit rows, when the caller has made them (as columns of a wider product)."""
+        projection's 32-bit rows (biases added, `in_bias`), when the caller has made them (as columns of a wider product)."""
         n, ws, H, D, V = h.shape[0], ctx.workspace, self.n_head, self.head_dim, self.value_dim
         group = ctx.groups[cache.group]
         if proj is None:
             proj = ws.get("scored_in", (n, self.in_weight.shape[0]), torch.float32)
-            linear(h, self.in_weight, None, out=proj)
+            linear(h, self.in_weight, self.in_bias, out=proj)
         P = self.row_dim
         q = ws.get("scored_q", (n, H * (P or D)), self.dtype)
         if not writes_cache:
             raise Unsupported("scored attention: a run that reads another run's cache is not supported")
         ops.qk_prepare(proj, q, cache.k, cache.v, group.slots, ctx.positions, q_off=self.q_off, k_off=self.k_off, v_off=self.v_off,
                        n_head=H, q_norm=self.q_norm, k_norm=self.k_norm, eps=self.eps, freqs=self.freqs, rot_dims=self.rot_dims,
-                       temp_coef=self.temp_coef, temp_every=self.temp_every, head_dim=D, value_dim=V)
+                       temp_coef=self.temp_coef, temp_every=self.temp_every, head_dim=D, value_dim=V, rot_halves=self.rot_halves,
+                       rot_mag=self.rot_mag, **self._shared_values(ws, n))
         att = ws.get("scored_att", (n, H * (P or V)), self.dtype)
         gate = proj[:, self.gate_off:self.gate_off + H * V] if self.gated else None
         if D == V or P:
             # keys and values of one width: the paged attention kernels of the engine (tiles of a prompt's queries on the matrix
             # cores, single tokens in splits, the 32-bit form), which cap and bias the scores when asked to
             splits = ops.attention(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, window=self.window,
-                                   softcap=self.softcap, bias_table=self.bias_table)
+                                   softcap=self.softcap, bias_table=self.bias_table, sinks=self.sinks)
             assert splits is None
             if gate is not None:
                 ops.gate_rows(att, gate)
         else:
             ops.attention_scored(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, softcap=self.softcap,
-                                 window=self.window, bias_table=self.bias_table, gate=gate)
+                                 window=self.window, bias_table=self.bias_table, gate=gate, sinks=self.sinks)
         if out is not None:
             linear(att, self.out_weight, None, out=out)
         else:

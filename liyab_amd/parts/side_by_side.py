@@ -15,7 +15,7 @@ from .registry import build_part, register_mixer
 
 class SideBySide:
     """result = weight * (left(h) / rms(left(h)) * w_left + right(h) / rms(right(h)) * w_right), the root mean squares over
-    the model's width. The two mixers are parts of the mixer registry that can leave their result to the caller
+    the model's width; or, for a spec that is not `normed`, left_weight * left(h) + right_weight * right(h). The two mixers are parts of the mixer registry that can leave their result to the caller
     (`forward(..., out=)`); at most one of them keeps rows in the pages and at most one keeps state, and this part passes
     the layer's cache and slot on to the one that does."""
 
@@ -38,16 +38,23 @@ class SideBySide:
         if self.left.state_spec() is not None and self.right.state_spec() is not None:
             raise ValueError("mixers side by side: only one of them may keep state")
         t = spec.tensors
-        self.left_out = store.fetch(t["left_out"], (self.width,), "vector")
-        self.right_out = store.fetch(t["right_out"], (self.width,), "vector")
+        self.normed = bool(getattr(spec, "normed", True))
+        self.left_weight, self.right_weight = float(getattr(spec, "left_weight", 1.0)), float(getattr(spec, "right_weight", 1.0))
+        self.left_out = store.fetch(t["left_out"], (self.width,), "vector") if self.normed else None
+        self.right_out = store.fetch(t["right_out"], (self.width,), "vector") if self.normed else None
         # both read the same rows: where both have one input projection and take its rows from the caller (`in_weight`,
         # forward(..., proj=)), the two run as one product [left | right]
-        self.joint_weight = None
+        self.joint_weight = self.joint_bias = None
         if all(isinstance(getattr(p, "in_weight", None), torch.Tensor) and "proj" in p.forward.__code__.co_varnames for p in (self.left, self.right)) \
                 and self.left.in_weight.dtype == self.right.in_weight.dtype:
             lw, rw = self.left.in_weight, self.right.in_weight
             self.joint_weight = store.derived(("joined_rows", id(lw), id(rw)), lambda: torch.cat([lw, rw], dim=0).contiguous())
             self.left_cols = lw.shape[0]
+            lb, rb = getattr(self.left, "in_bias", None), getattr(self.right, "in_bias", None)
+            if lb is not None or rb is not None:
+                zeros = lambda rows: torch.zeros(rows, dtype=torch.float32, device=lw.device)  # noqa: E731
+                self.joint_bias = store.derived(("joined_bias", id(lw), id(rw)), lambda: torch.cat(
+                    [lb if lb is not None else zeros(lw.shape[0]), rb if rb is not None else zeros(rw.shape[0])]).contiguous())
         planners = [p for p in (getattr(self.left, "step_planner", None), getattr(self.right, "step_planner", None)) if p is not None]
         if len(planners) > 1:
             raise ValueError("mixers side by side: only one of them may plan a step")
@@ -67,13 +74,19 @@ class SideBySide:
         b = ws.get("side_right", (n, self.width), torch.float32)
         if self.joint_weight is not None:
             proj = ws.get("side_in", (n, self.joint_weight.shape[0]), torch.float32)
-            linear(h, self.joint_weight, None, out=proj)
+            linear(h, self.joint_weight, self.joint_bias, out=proj)
             self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=a, proj=proj[:, :self.left_cols])
             self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=b, proj=proj[:, self.left_cols:])
         else:
             self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=a)
             self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=b)
-        if out is not None:
+        if not self.normed:
+            if out is not None:
+                ops.weighted_sum(out, a, b, self.left_weight, self.right_weight)
+            else:
+                ops.weighted_sum(a, a, b, self.left_weight, self.right_weight)
+                ops.add_into_(settled(residual), a)
+        elif out is not None:
             ops.fill_(out, 0)
             ops.mean_norm_add(out, a, b, self.left_out, self.right_out, self.eps, self.weight)
         else:
