@@ -5,7 +5,7 @@
 // (values may be the keys' own columns: values that are the keys as projected). Per head, in this
 // order: a root-mean-square norm over the head with a weight shared by all heads (queries and keys,
 // each optional); the turning of pairs of the first `rot_dims` entries by position * f_i (queries and keys; f from a
-// table; pairs (2i, 2i + 1), or (i, i + rot_dims / 2) with `rot_halves`; cosine and sine times `rot_mag`); a factor on the query that grows with the logarithm of the
+// table of doubles; pairs (2i, 2i + 1), or (i, i + rot_dims / 2) with `rot_halves`; cosine and sine times `rot_mag`); a factor on the query that grows with the logarithm of the
 // position, 1 + coef * ln(floor((p + 1) / every) + 1). Queries go to a dense buffer in the compute type,
 // keys and values to their token's slot of the pages; the rows they go to may be wider than the heads (dk_out, dv_out),
 // zeros behind them: keys and values padded to one width are what the matrix-core kernels take. Norms, angles and factors are 32-bit.
@@ -25,12 +25,20 @@ namespace liyab {
 
 constexpr int AS_THREADS = 256;
 
+// position * frequency, taken in double precision and brought into [0, 2 pi) before it is rounded: at position 1,000 a 32-bit
+// product is already off by 6e-5 of a turn's radian, which is more than every other rounding of a 32-bit row together
+__device__ __forceinline__ float turn_angle(int p, double f) {
+    const double a = static_cast<double>(p) * f;
+    constexpr double kTwoPi = 6.283185307179586476925286766559;
+    return static_cast<float>(a - kTwoPi * floor(a / kTwoPi));
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kWave)
 qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, int dk_out,
                   int dv_out, T* __restrict__ q_out, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots, int page_size,
                   int num_pages, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps,
-                  const float* __restrict__ freqs, int rot_dims, float temp_coef, int temp_every, const int* __restrict__ positions,
+                  const double* __restrict__ freqs, int rot_dims, float temp_coef, int temp_every, const int* __restrict__ positions,
                   int rot_halves, float rot_mag, float* __restrict__ v_keep, const float* __restrict__ v_first, const float* __restrict__ v_lam) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
     const int p = positions[t];
@@ -63,7 +71,7 @@ qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_of
             for (int i = lane; i < half; i += kWave) {
                 const float a = x[i] * factor * (nw != nullptr ? nw[i] : 1.0f);
                 const float b = x[i + half] * factor * (nw != nullptr ? nw[i + half] : 1.0f);
-                const float angle = static_cast<float>(p) * freqs[i];
+                const float angle = turn_angle(p, freqs[i]);
                 const float c = cosf(angle) * rot_mag, s = sinf(angle) * rot_mag;
                 dst[i] = from_float<T>((a * c - b * s) * temp);
                 dst[i + half] = from_float<T>((b * c + a * s) * temp);
@@ -77,7 +85,7 @@ qk_prepare_kernel(const float* __restrict__ src, int64_t ld, int q_off, int k_of
             float a = x[e0] * factor * (nw != nullptr ? nw[e0] : 1.0f);
             float b = e1 < dk ? x[e1] * factor * (nw != nullptr ? nw[e1] : 1.0f) : 0.0f;
             if (freqs != nullptr && e1 < rot_dims) {
-                const float angle = static_cast<float>(p) * freqs[i2];
+                const float angle = turn_angle(p, freqs[i2]);
                 const float c = cosf(angle) * rot_mag, s = sinf(angle) * rot_mag;
                 const float ra = a * c - b * s, rb = b * c + a * s;
                 a = ra;
@@ -202,7 +210,7 @@ using namespace liyab;
 
 extern "C" int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, int dk_out,
                                 int dv_out, void* q_out, void* kc, void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm,
-                                const float* k_norm, float eps, const float* freqs, int rot_dims, float temp_coef, int temp_every,
+                                const float* k_norm, float eps, const double* freqs, int rot_dims, float temp_coef, int temp_every,
                                 const int* positions, int n, int rot_halves, float rot_mag, float* v_keep, const float* v_first,
                                 const float* v_lam, hipStream_t stream) {
     LIYAB_REQUIRE(src && q_out && kc && vc && slots && positions, "qk_prepare: null pointer");
@@ -217,7 +225,7 @@ extern "C" int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_o
     LIYAB_REQUIRE((v_first == nullptr) == (v_lam == nullptr) && !(v_keep != nullptr && v_first != nullptr), "qk_prepare: values are kept, or mixed with kept ones and a rate");
     if (n == 0) return 0;
     dim3 grid(n, H + 2 * G);
-    const float* fr = rot_dims > 0 ? freqs : nullptr;
+    const double* fr = rot_dims > 0 ? freqs : nullptr;
     if (dtype == kF32)
         qk_prepare_kernel<float><<<grid, kWave, 0, stream>>>(src, ld, q_off, k_off, v_off, H, G, dk, dv, dk_out, dv_out, static_cast<float*>(q_out), static_cast<float*>(kc),
                                                              static_cast<float*>(vc), slots, page_size, num_pages, q_norm, k_norm, eps, fr, rot_dims,

@@ -120,7 +120,7 @@ int liyab_gated_group_norm(void* out, int out_dtype, const float* y, int64_t ldy
                            int n, int inner, int groups, hipStream_t stream);
 int liyab_qk_prepare(const float* src, int64_t ld, int q_off, int k_off, int v_off, int H, int G, int dk, int dv, int dk_out, int dv_out,
                      void* q_out, void* kc, void* vc, int dtype, const int* slots, int page_size, int num_pages, const float* q_norm, const float* k_norm,
-                     float eps, const float* freqs, int rot_dims, float temp_coef, int temp_every, const int* positions, int n,
+                     float eps, const double* freqs, int rot_dims, float temp_coef, int temp_every, const int* positions, int n,
                      int rot_halves, float rot_mag, float* v_keep, const float* v_first, const float* v_lam, hipStream_t stream);
 int liyab_attention_scored(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* kc, const void* vc, int dtype,
                            const int* block_tables, int max_blocks, const int* tok_seq, const int* tok_pos, int n, float scale,

@@ -1545,7 +1545,7 @@ def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_
     """From a projection's float32 rows `src` (queries at column q_off, keys at k_off, values at v_off, which may be k_off) to
     queries in `q_out` [n, heads * dk] and keys and values in their slots of the pages (k_cache [pages, kv_heads, page, dk],
     v_cache [.., dv]), all in the compute dtype. Per head, each optional: a root-mean-square norm with a weight [dk] (queries,
-    keys), pairs (2i, 2i + 1) of the first rot_dims entries turned by position * freqs[i] (queries, keys), the query times
+    keys), pairs (2i, 2i + 1) of the first rot_dims entries turned by position * freqs[i] (queries, keys; freqs float64), the query times
     1 + temp_coef * ln(floor((position + 1) / temp_every) + 1). A slot outside the pages is not written. `head_dim`,
     `value_dim`: the heads' own widths where the caches' rows (and the queries') are wider, zeros behind the heads. `rot_halves`:
     the turned pairs are (i, i + rot_dims / 2) instead; `rot_mag` multiplies cosine and sine. `v_keep` (float32 [n, kv_heads * dv]) gets
@@ -1572,7 +1572,9 @@ def qk_prepare(src: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_
     if rot_dims:
         if rot_dims % 2 or rot_dims > dk or freqs is None:
             raise KernelError(f"qk_prepare: {rot_dims} turned entries of heads of {dk}")
-        _f32vec(freqs, "freqs", rot_dims // 2)
+        _dev(freqs, "freqs")
+        if freqs.dtype != torch.float64 or not freqs.is_contiguous() or freqs.numel() != rot_dims // 2:
+            raise KernelError(f"qk_prepare: the frequencies must be {rot_dims // 2} contiguous float64 values")
     _i32(slots, "slots", n)
     _i32(positions, "positions", n)
     for kept, what in ((v_keep, "v_keep"), (v_first, "v_first")):

@@ -146,7 +146,7 @@ class ScoredAttention:
             self.rot_dims = int(rot.dims)
             self.rot_halves, self.rot_mag = bool(getattr(rot, "halves", False)), rotary_magnitude(rot)
             self.freqs = store.derived(("rotary", rot.dims, rot.base, rot.scaling, getattr(rot, "ramp", None)),
-                                       lambda: torch.from_numpy(rotary_frequencies(rot).astype(np.float32)).to(self.out_weight.device))
+                                       lambda: torch.from_numpy(rotary_frequencies(rot).astype(np.float64)).to(self.out_weight.device))
         self.temp_coef, self.temp_every = (float(spec.q_temp[0]), int(spec.q_temp[1])) if spec.q_temp else (0.0, 0)
         self.bias_table = None
         if spec.distance_bias:
