@@ -10,7 +10,7 @@
 //
 // liyab_activate: tanh, silu, the logistic function or the squared positive part of 32-bit rows, rounded to the output type.
 //
-// liyab_gate_rows: x *= sigmoid(g) in place, a gate on a mixer's rows from 32-bit logits.
+// liyab_gate_rows: x *= scale * sigmoid(g) in place, a gate on a mixer's rows from 32-bit logits (and a constant factor).
 //
 // liyab_mean_norm_add: x += weight * (a / rms(a) * wa + b / rms(b) * wb), the two results of
 // sublayers that run side by side, each brought to unit root mean square over the row first.
@@ -69,12 +69,12 @@ activate_kernel(T* __restrict__ out, int64_t ldo, const float* __restrict__ in, 
 
 template <typename T>
 __global__ void __launch_bounds__(EW_THREADS)
-gate_rows_kernel(T* __restrict__ x, int64_t ldx, const float* __restrict__ gate, int64_t ldg, int d) {
+gate_rows_kernel(T* __restrict__ x, int64_t ldx, const float* __restrict__ gate, int64_t ldg, int d, float scale) {
     const int t = blockIdx.y;
     const int i = blockIdx.x * EW_THREADS + threadIdx.x;
     if (i >= d) return;
     T* at = x + static_cast<int64_t>(t) * ldx + i;
-    *at = from_float<T>(to_float<T>(*at) * logistic(gate[static_cast<int64_t>(t) * ldg + i]));
+    *at = from_float<T>(to_float<T>(*at) * logistic(gate[static_cast<int64_t>(t) * ldg + i]) * scale);
 }
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
@@ -159,14 +159,14 @@ extern "C" int liyab_activate(void* out, int out_dtype, int64_t ldo, const float
     return check_launch("activate");
 }
 
-// x[t, i] *= sigmoid(gate[t, i]) in place; x rows in float32 or bfloat16, gate float32 logits.
-extern "C" int liyab_gate_rows(void* x, int dtype, int64_t ldx, const float* gate, int64_t ldg, int n, int d, hipStream_t stream) {
+// x[t, i] *= scale * sigmoid(gate[t, i]) in place; x rows in float32 or bfloat16, gate float32 logits.
+extern "C" int liyab_gate_rows(void* x, int dtype, int64_t ldx, const float* gate, int64_t ldg, int n, int d, float scale, hipStream_t stream) {
     LIYAB_REQUIRE(x && gate, "gate_rows: null pointer");
     LIYAB_REQUIRE(n >= 0 && n <= 65535 && d > 0 && ldx >= d && ldg >= d, "gate_rows: bad sizes");
     if (n == 0) return 0;
     dim3 grid((d + EW_THREADS - 1) / EW_THREADS, n);
-    if (dtype == kF32) gate_rows_kernel<float><<<grid, EW_THREADS, 0, stream>>>(static_cast<float*>(x), ldx, gate, ldg, d);
-    else if (dtype == kBF16) gate_rows_kernel<bf16_t><<<grid, EW_THREADS, 0, stream>>>(static_cast<bf16_t*>(x), ldx, gate, ldg, d);
+    if (dtype == kF32) gate_rows_kernel<float><<<grid, EW_THREADS, 0, stream>>>(static_cast<float*>(x), ldx, gate, ldg, d, scale);
+    else if (dtype == kBF16) gate_rows_kernel<bf16_t><<<grid, EW_THREADS, 0, stream>>>(static_cast<bf16_t*>(x), ldx, gate, ldg, d, scale);
     else return fail(1, "gate_rows: unknown dtype %d", dtype);
     return check_launch("gate_rows");
 }

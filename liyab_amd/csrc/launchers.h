@@ -63,7 +63,7 @@ int liyab_rmsnorm(void* out, int out_dtype, const float* x, const float* w, cons
 int liyab_gated_norm_add(float* x, void* cast_out, int cast_dtype, const float* y, int n_sum, const float* gate, int64_t gate_stride,
                          const float* w, float eps, int normalize, int n, int d, float* state, int ring, int n_slots,
                          const int* tok_seq, const int* positions, const int* context_lens, const int* state_slots, const int* n_real,
-                         hipStream_t stream);
+                         const float* next_w, float next_eps, hipStream_t stream);
 int liyab_causal_conv(void* out, void* cast_out, int dtype, const float* x, const float* w, int taps, const float* state, int n_slots,
                       const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots, int n, int d,
                       hipStream_t stream);
@@ -91,7 +91,7 @@ int liyab_attention_prefill_scored(void* out, int64_t out_stride, const void* q,
                                    const int* block_tables, int max_blocks, const int* work, int n_tiles, int tile, int ksplit, float scale,
                                    int window, int n_head, int n_kv_head, int hd, int page_size, int num_pages, float softcap,
                                    const float* bias_table, int max_dist, const float* sinks, hipStream_t stream);
-int liyab_gate_rows(void* x, int dtype, int64_t ldx, const float* gate, int64_t ldg, int n, int d, hipStream_t stream);
+int liyab_gate_rows(void* x, int dtype, int64_t ldx, const float* gate, int64_t ldg, int n, int d, float scale, hipStream_t stream);
 int liyab_dyt(void* out, int out_dtype, const float* x, const float* w, const float* b, const float* alpha, const int* rows, int n, int d,
               hipStream_t stream);
 int liyab_glu_clamped(void* out, int out_dtype, const float* gu, int64_t ld, int n, int ff, float limit, float slope, float shift,
@@ -156,10 +156,14 @@ int liyab_maps_join(void* out, const void* a1, const void* a2, int64_t lda, int 
 
 
 int liyab_weighted_sum(float* out, const float* a, const float* b, float wa, float wb, int64_t n, hipStream_t stream);
-int liyab_lru_gates(float* decay, float* input, const float* u, int64_t ldu, const void* wr, const void* wi, int w_dtype, const float* br,
-                    const float* bi, const float* lam, float rate, int n, int blocks, int width, hipStream_t stream);
-int liyab_lru_scan(void* out, int out_dtype, const float* decay, const float* input, const float* y, int64_t ldy, float* state,
-                   int64_t state_stride, int n_slots, const int* seq_starts, const int* positions, const int* state_slots, int n_seqs,
-                   int width, hipStream_t stream);
+int liyab_lru_conv(float* out, void* split, const float* in, int64_t ldi, const float* w, const float* bias, int taps, const float* state,
+                   int64_t state_stride, int n_slots, const int* tok_seq, const int* positions, const int* seq_starts, const int* state_slots,
+                   int n, int C, int blocks, hipStream_t stream);
+int liyab_lru_coeffs(float* decay, float* gated, const float* z, int64_t ldz, const float* u, const float* br, const float* bi, const float* lam,
+                     float rate, int n, int C, int blocks, hipStream_t stream);
+int liyab_lru_scan(void* out, int out_dtype, const float* z, int64_t ldz, const float* u, const float* decay, const float* gated, const float* br,
+                   const float* bi, const float* lam, float rate, float out_scale, const float* y, int64_t ldy, float* state,
+                   int64_t state_stride, int n_slots, const float* x, int64_t ldx, int taps, const int* seq_starts, const int* positions,
+                   const int* state_slots, int n_seqs, int C, int blocks, int stretches, hipStream_t stream);
 
 }  // extern "C"

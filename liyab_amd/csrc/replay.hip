@@ -122,7 +122,8 @@ static const Entry kEntries[] = {
     LIYAB_ENTRY(liyab_maps_store),
     LIYAB_ENTRY(liyab_maps_join),
     LIYAB_ENTRY(liyab_weighted_sum),
-    LIYAB_ENTRY(liyab_lru_gates),
+    LIYAB_ENTRY(liyab_lru_conv),
+    LIYAB_ENTRY(liyab_lru_coeffs),
     LIYAB_ENTRY(liyab_lru_scan),
 };
 constexpr int kNumEntries = static_cast<int>(sizeof(kEntries) / sizeof(kEntries[0]));

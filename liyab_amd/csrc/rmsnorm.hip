@@ -11,7 +11,8 @@
 // without `normalize` the sum is added as it is (x += s);
 // g: the gate's 32-bit logits (a pointer and a row stride, so that they may be columns of a wider
 // product), or none. The new row may also be written rounded to the compute type for the next
-// product (`cast_out`). Before a row is updated it may be kept as the request's input history of
+// product (`cast_out`), or, with `next_w`, what the next sublayer reads of it: the new row's own root-mean-square norm under that
+// weight and `next_eps` (a block with a norm before its sublayers as well as behind them). Before a row is updated it may be kept as the request's input history of
 // a causal convolution over time: `state` [slots, ring, d] holds position p at ring place p % ring,
 // and the last `ring` rows of each request in the step are the ones that a later step reads.
 #include "common.h"
@@ -70,7 +71,8 @@ __device__ __forceinline__ float sigmoidf(float z) { return 1.0f / (1.0f + expf(
 template <typename T, int THREADS, int MAXV>
 __global__ void __launch_bounds__(THREADS)
 gated_norm_add_kernel(float* __restrict__ x, T* __restrict__ cast_out, const float* __restrict__ y, int n_sum,
-                      const float* __restrict__ gate, int64_t gate_stride, const float* __restrict__ w, float eps, int normalize, int d, KeepRows keep) {
+                      const float* __restrict__ gate, int64_t gate_stride, const float* __restrict__ w, float eps, int normalize, int d, KeepRows keep,
+                      const float* __restrict__ next_w, float next_eps) {
     __shared__ float red[THREADS / kWave];
     const int t = blockIdx.x;
     float* xr = x + static_cast<int64_t>(t) * d;
@@ -108,21 +110,37 @@ gated_norm_add_kernel(float* __restrict__ x, T* __restrict__ cast_out, const flo
     }
     const float scale = normalize ? 1.0f / sqrtf(rms_block_sum<THREADS>(ss, red) / static_cast<float>(d) + eps) : 1.0f;
     T* co = cast_out != nullptr ? cast_out + static_cast<int64_t>(t) * d : nullptr;
+    const bool norm_next = next_w != nullptr && co != nullptr;  // what is written for the next product is the next norm of the new row
+    float ss_new = 0.0f;
     auto finish = [&](int i, float s) {
         float v = s * scale;
         if (w != nullptr) v *= w[i];
         v += xr[i];
         xr[i] = v;
-        if (co != nullptr) co[i] = from_float<T>(v);
+        if (norm_next) ss_new += v * v;
+        else if (co != nullptr) co[i] = from_float<T>(v);
+        return v;
     };
     if (held) {
 #pragma unroll
         for (int j = 0; j < MAXV; ++j) {
             const int i = threadIdx.x + j * THREADS;
-            if (i < d) finish(i, sv[j]);
+            if (i < d) sv[j] = finish(i, sv[j]);
         }
     } else {
         for (int i = threadIdx.x; i < d; i += THREADS) finish(i, value(i));
+    }
+    if (norm_next) {
+        const float next_scale = 1.0f / sqrtf(rms_block_sum<THREADS>(ss_new, red) / static_cast<float>(d) + next_eps);
+        if (held) {
+#pragma unroll
+            for (int j = 0; j < MAXV; ++j) {
+                const int i = threadIdx.x + j * THREADS;
+                if (i < d) co[i] = from_float<T>(sv[j] * next_scale * next_w[i]);
+            }
+        } else {
+            for (int i = threadIdx.x; i < d; i += THREADS) co[i] = from_float<T>(xr[i] * next_scale * next_w[i]);  // (each thread reads what it wrote)
+        }
     }
 }
 
@@ -146,8 +164,9 @@ extern "C" int liyab_rmsnorm(void* out, int out_dtype, const float* x, const flo
 extern "C" int liyab_gated_norm_add(float* x, void* cast_out, int cast_dtype, const float* y, int n_sum, const float* gate,
                                     int64_t gate_stride, const float* w, float eps, int normalize, int n, int d, float* state, int ring, int n_slots,
                                     const int* tok_seq, const int* positions, const int* context_lens, const int* state_slots,
-                                    const int* n_real, hipStream_t stream) {
+                                    const int* n_real, const float* next_w, float next_eps, hipStream_t stream) {
     LIYAB_REQUIRE(x && y, "gated_norm_add: null pointer");
+    LIYAB_REQUIRE(next_w == nullptr || cast_out != nullptr, "gated_norm_add: the next norm's rows need a place");
     LIYAB_REQUIRE(n >= 0 && d > 0 && n_sum >= 1, "gated_norm_add: bad sizes n=%d d=%d n_sum=%d", n, d, n_sum);
     LIYAB_REQUIRE(cast_dtype == kF32 || cast_dtype == kBF16, "gated_norm_add: unknown dtype %d", cast_dtype);
     LIYAB_REQUIRE(gate == nullptr || gate_stride >= d, "gated_norm_add: the gate's row stride is shorter than a row");
@@ -156,8 +175,8 @@ extern "C" int liyab_gated_norm_add(float* x, void* cast_out, int cast_dtype, co
     if (n == 0) return 0;
     const KeepRows keep{state, ring, n_slots, tok_seq, positions, context_lens, state_slots, n_real};
     if (cast_dtype == kF32)
-        gated_norm_add_kernel<float, 256, 8><<<n, 256, 0, stream>>>(x, static_cast<float*>(cast_out), y, n_sum, gate, gate_stride, w, eps, normalize, d, keep);
+        gated_norm_add_kernel<float, 256, 8><<<n, 256, 0, stream>>>(x, static_cast<float*>(cast_out), y, n_sum, gate, gate_stride, w, eps, normalize, d, keep, next_w, next_eps);
     else
-        gated_norm_add_kernel<bf16_t, 256, 8><<<n, 256, 0, stream>>>(x, static_cast<bf16_t*>(cast_out), y, n_sum, gate, gate_stride, w, eps, normalize, d, keep);
+        gated_norm_add_kernel<bf16_t, 256, 8><<<n, 256, 0, stream>>>(x, static_cast<bf16_t*>(cast_out), y, n_sum, gate, gate_stride, w, eps, normalize, d, keep, next_w, next_eps);
     return check_launch("gated_norm_add");
 }

@@ -74,7 +74,7 @@ _SIGNATURES = {
     "liyab_argmax_static": [P, P, c_int64, c_int, c_int, P, P, P],
     "liyab_sample": [P, P, c_int64, c_int, c_int, P, P, P, P, P, P, P],
     "liyab_rmsnorm": [P, c_int, P, P, P, c_int, c_int, c_float, P],
-    "liyab_gated_norm_add": [P, P, c_int, P, c_int, P, c_int64, P, c_float, c_int, c_int, c_int, P, c_int, c_int, P, P, P, P, P, P],
+    "liyab_gated_norm_add": [P, P, c_int, P, c_int, P, c_int64, P, c_float, c_int, c_int, c_int, P, c_int, c_int, P, P, P, P, P, P, c_float, P],
     "liyab_causal_conv": [P, P, c_int, P, P, c_int, P, c_int, P, P, P, P, c_int, c_int, P],
     "liyab_keep_rows": [P, c_int, c_int, P, P, P, P, P, P, c_int, c_int, P],
     "liyab_latent_store": [P, c_int, P, c_int64, c_int, P, c_float, P, c_int, c_int, c_int, c_int, P],
@@ -87,7 +87,7 @@ _SIGNATURES = {
                                       c_int, c_int, c_int, c_int, c_int, c_int, P, c_int, c_int, c_float, P, c_int, P, P],
     "liyab_attention_prefill_scored": [P, c_int64, P, c_int64, P, P, P, c_int, P, c_int, c_int, c_int, c_float, c_int, c_int,
                                        c_int, c_int, c_int, c_int, c_float, P, c_int, P, P],
-    "liyab_gate_rows": [P, c_int, c_int64, P, c_int64, c_int, c_int, P],
+    "liyab_gate_rows": [P, c_int, c_int64, P, c_int64, c_int, c_int, c_float, P],
     "liyab_dyt": [P, c_int, P, P, P, P, P, c_int, c_int, P],
     "liyab_glu_clamped": [P, c_int, P, c_int64, c_int, c_int, c_float, c_float, c_float, P],
     "liyab_activate": [P, c_int, c_int64, P, c_int64, c_int, c_int, c_int, P],
@@ -116,8 +116,10 @@ _SIGNATURES = {
                          c_int, c_int, c_int, c_int, P],
     "liyab_maps_join": [P, P, P, c_int64, c_int, c_float, c_float, c_float, c_int, c_int, c_int, c_int, P],
     "liyab_weighted_sum": [P, P, P, c_float, c_float, c_int64, P],
-    "liyab_lru_gates": [P, P, P, c_int64, P, P, c_int, P, P, P, c_float, c_int, c_int, c_int, P],
-    "liyab_lru_scan": [P, c_int, P, P, P, c_int64, P, c_int64, c_int, P, P, P, c_int, c_int, P],
+    "liyab_lru_conv": [P, P, P, c_int64, P, P, c_int, P, c_int64, c_int, P, P, P, P, c_int, c_int, c_int, P],
+    "liyab_lru_coeffs": [P, P, P, c_int64, P, P, P, P, c_float, c_int, c_int, c_int, P],
+    "liyab_lru_scan": [P, c_int, P, c_int64, P, P, P, P, P, P, c_float, c_float, P, c_int64, P, c_int64, c_int, P, c_int64, c_int, P, P, P, c_int, c_int,
+                       c_int, c_int, P],
 }
 
 

@@ -1086,13 +1086,14 @@ def _keep_args(keep, d: int):
 
 def gated_norm_add(x: torch.Tensor, y: torch.Tensor, weight: Optional[torch.Tensor], eps: float, *, n_sum: int = 1,
                    gate: Optional[torch.Tensor] = None, cast_out: Optional[torch.Tensor] = None, keep=None,
-                   normalize: bool = True) -> None:
+                   normalize: bool = True, next_norm=None) -> None:
     """x[t] += weight * s / sqrt(mean(s^2) + eps) with s = (y[t * n_sum] + ... + y[t * n_sum + n_sum - 1]) *
     sigmoid(gate[t]); x float32 [n, d] in place, y float32 [n * n_sum, d], gate float32 [n, d] (rows may
     be strided: columns of a wider product) or None. `cast_out` [n, d] (float32 or bfloat16) gets the new
     rows rounded. `keep` = (state, ctx): before the update, the last rows of each request go to its input
     history, state[slot, position % ring] (the rows behind the step's tokens are left out). Without
-    `normalize`: x[t] += s."""
+    `normalize`: x[t] += s. `next_norm` = (weight float32 [d], eps): `cast_out` gets the new row's root-mean-square norm under
+    that weight instead of the row itself (what the next sublayer reads)."""
     _dev(x, "x")
     _dev(y, "y")
     n, d = x.shape
@@ -1114,8 +1115,12 @@ def gated_norm_add(x: torch.Tensor, y: torch.Tensor, weight: Optional[torch.Tens
         code = dtype_code(cast_out.dtype)
     if keep is not None and keep[1].n_tokens != n:
         raise KernelError("gated_norm_add: rows are kept for a step of as many rows as x has")
+    next_w, next_eps = (None, 0.0) if next_norm is None else next_norm
+    _f32vec(next_w, "the next norm's weight", d)
+    if next_w is not None and cast_out is None:
+        raise KernelError("gated_norm_add: the next norm's rows need a place (cast_out)")
     _lib.call("liyab_gated_norm_add", x.data_ptr(), _ptr(cast_out), code, y.data_ptr(), n_sum, _ptr(gate), gs, _ptr(weight), float(eps),
-              1 if normalize else 0, n, d, *_keep_args(keep, d), _stream())
+              1 if normalize else 0, n, d, *_keep_args(keep, d), _ptr(next_w), float(next_eps), _stream())
 
 
 def keep_rows(x: torch.Tensor, state: torch.Tensor, ctx) -> None:
@@ -1629,13 +1634,13 @@ def attention_scored(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, 
               int(window), _ptr(bias_table), max_dist, _ptr(gate), gs, n_head, G, dk, dv, page, _pages(k_cache, num_pages), _ptr(sinks), _stream())
 
 
-def gate_rows(x: torch.Tensor, gate: torch.Tensor) -> None:
-    """x *= sigmoid(gate) in place; x rows in float32 or bfloat16, gate float32 rows of the same shape (columns of wider
+def gate_rows(x: torch.Tensor, gate: torch.Tensor, scale: float = 1.0) -> None:
+    """x *= scale * sigmoid(gate) in place; x rows in float32 or bfloat16, gate float32 rows of the same shape (columns of wider
     rows are fine)."""
     ldx, ldg = _rows(x, "x"), _rows(gate, "gate")
     if gate.dtype != torch.float32 or gate.shape != x.shape:
         raise KernelError("gate_rows: the gate must be float32 and of x's shape")
-    _lib.call("liyab_gate_rows", x.data_ptr(), dtype_code(x.dtype), ldx, gate.data_ptr(), ldg, x.shape[0], x.shape[1], _stream())
+    _lib.call("liyab_gate_rows", x.data_ptr(), dtype_code(x.dtype), ldx, gate.data_ptr(), ldg, x.shape[0], x.shape[1], float(scale), _stream())
 
 
 # -- two norms of one stream with a convolution over time each; rings of kept rows; small row kernels ---------
@@ -1877,44 +1882,77 @@ def weighted_sum(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, wa: float,
     _lib.call("liyab_weighted_sum", out.data_ptr(), a.data_ptr(), b.data_ptr(), float(wa), float(wb), out.numel(), _stream())
 
 
-def lru_gates(decay: torch.Tensor, gated: torch.Tensor, u: torch.Tensor, wr: torch.Tensor, wi: torch.Tensor, br: torch.Tensor, bi: torch.Tensor,
-              lam: torch.Tensor, rate: float) -> None:
-    """From the recurrence's input u (float32 rows [n, width], columns of wider rows are fine) in `blocks` equal parts: r = sigmoid(Wr[b]
-    u_b + br), i = sigmoid(Wi[b] u_b + bi), decay = exp(-rate * r * softplus(lam)), gated = sqrt(1 - decay^2) * i * u; decay and gated
-    contiguous float32 [n, width]. wr, wi [blocks, in, out] (a part's matrix transposed), bfloat16 or float32; br, bi, lam float32 [width]."""
-    ldu = _rows(u, "u")
-    n, W = u.shape
-    _dev(wr, "wr")
-    if wr.dim() != 3 or wr.shape[1] != wr.shape[2] or wr.shape[0] * wr.shape[1] != W or wr.shape != wi.shape or wr.dtype != wi.dtype \
-            or not wr.is_contiguous() or not wi.is_contiguous():
-        raise KernelError(f"lru_gates: the gates' matrices must be contiguous [blocks, in, out] over {W} channels, got {tuple(wr.shape)} / {tuple(wi.shape)}")
-    if u.dtype != torch.float32:
-        raise KernelError("lru_gates: u must be float32")
-    for t, what in ((decay, "decay"), (gated, "gated")):
-        _dev(t, what)
-        if t.dtype != torch.float32 or tuple(t.shape) != (n, W) or not t.is_contiguous():
-            raise KernelError(f"lru_gates: {what} must be contiguous float32 [{n}, {W}]")
-    _f32vec(br, "br", W)
-    _f32vec(bi, "bi", W)
-    _f32vec(lam, "lam", W)
-    _lib.call("liyab_lru_gates", decay.data_ptr(), gated.data_ptr(), u.data_ptr(), ldu, wr.data_ptr(), wi.data_ptr(), dtype_code(wr.dtype), br.data_ptr(),
-              bi.data_ptr(), lam.data_ptr(), float(rate), n, wr.shape[0], W, _stream())
+def lru_conv(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor], ring_off: int,
+             ctx, blocks: int = 1, split: Optional[torch.Tensor] = None) -> None:
+    """out[t, c] = bias[c] + sum_j weight[c, j] * x[t - taps + 1 + j, c] over each request's own rows in time; x float32 rows (columns of
+    wider rows are fine), out contiguous float32 [n, C], weight float32 [C, taps]; the rows before a request's first row of the step come
+    from state[slot, ring_off + (position % (taps - 1)) * C + c], zeros before position 0. `split` (bfloat16 [n, 2 C]): out once more as
+    two bfloat16 numbers a value, out = hi + lo, each of the `blocks` equal parts of the channels as [hi | lo]."""
+    ldi = _rows(x, "x")
+    n, C = x.shape
+    _dev(out, "out")
+    if x.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (n, C) or not out.is_contiguous() or ctx.n_tokens != n:
+        raise KernelError("lru_conv: x must be the step's float32 rows and out contiguous float32 of the same shape")
+    _dev(weight, "weight")
+    if weight.dtype != torch.float32 or weight.dim() != 2 or weight.shape[0] != C or not weight.is_contiguous():
+        raise KernelError(f"lru_conv: the weight must be contiguous float32 [{C}, taps]")
+    taps = weight.shape[1]
+    if not 1 <= taps <= CONV_MAX_TAPS or blocks < 1 or C % blocks:
+        raise KernelError(f"lru_conv: {taps} taps (1 to {CONV_MAX_TAPS}), {C} channels in {blocks} parts")
+    _f32vec(bias, "bias", C)
+    if split is not None:
+        _dev(split, "split")
+        if split.dtype != torch.bfloat16 or tuple(split.shape) != (n, 2 * C) or not split.is_contiguous():
+            raise KernelError(f"lru_conv: the split rows must be contiguous bfloat16 [{n}, {2 * C}]")
+    stride, slots, base = 0, 0, None
+    if taps > 1:
+        stride = _state(state, "lru_conv")
+        if ring_off < 0 or ring_off + (taps - 1) * C > stride:
+            raise KernelError("lru_conv: the ring does not lie in the slot")
+        slots, base = state.shape[0], state.data_ptr() + 4 * ring_off
+    _step_lists(ctx, n)
+    _lib.call("liyab_lru_conv", out.data_ptr(), _ptr(split), x.data_ptr(), ldi, weight.data_ptr(), _ptr(bias), taps, base, stride, slots,
+              ctx.tok_seq.data_ptr(), ctx.positions.data_ptr(), ctx.seq_starts.data_ptr(), ctx.state_slots.data_ptr(), n, C, int(blocks), _stream())
 
 
-def lru_scan(out: torch.Tensor, decay: torch.Tensor, gated: torch.Tensor, y: torch.Tensor, state: torch.Tensor, ctx) -> None:
-    """S_t = decay_t * S_(t-1) + gated_t along each request's rows of the step, from state[slot, :width] (zero at position 0), which gets
-    the last S; out[t] = S_t * gelu_tanh(y_t) in out's dtype. decay, gated float32 [n, width]; y float32 rows (columns of wider rows are
-    fine); out contiguous [n, width]."""
-    ldy = _rows(y, "y")
-    n, W = y.shape
+LRU_STRETCHES_FROM = 48  # the longest portion a step may hold from which its recurrence runs in stretches side by side
+
+
+def lru_stretches(ctx, n: int) -> bool:
+    """Whether a step's recurrence a channel runs in stretches side by side (sixteen waves a request, each a stretch of its rows) rather
+    than one wave a request: from the step's rows and requests alone, as its grids, so that a captured graph holds for every step of
+    its shape."""
+    return n - ctx.n_seqs + 1 >= LRU_STRETCHES_FROM
+
+
+def lru_scan(out: torch.Tensor, z: torch.Tensor, u: torch.Tensor, y: torch.Tensor, x: torch.Tensor, br: torch.Tensor, bi: torch.Tensor,
+             lam: torch.Tensor, rate: float, state: torch.Tensor, taps: int, ctx, blocks: int, out_scale: float = 1.0) -> None:
+    """S_t = a_t * S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t along each request's rows of the step, with r = sigmoid(zr + br), i = sigmoid(zi +
+    bi), a = exp(-rate * r * softplus(lam)); z float32 rows [n, 2 C], each of the `blocks` parts of the channels as [zr | zi]; u contiguous
+    float32 [n, C]. S starts from state[slot, :C] (zero at position 0), which gets the last S; out[t] = out_scale * S_t * gelu_tanh(y_t) in
+    out's dtype (y float32 rows, out contiguous [n, C]). The last taps - 1 rows of x (float32 rows) go to the slot's ring behind S,
+    position p at place p % (taps - 1). Steps that may hold a long portion walk in stretches (`lru_stretches`)."""
+    ldz, ldy, ldx = _rows(z, "z"), _rows(y, "y"), _rows(x, "x")
+    n, C = y.shape
     stride = _state(state, "lru_scan")
     _dev(out, "out")
-    if y.dtype != torch.float32 or tuple(out.shape) != (n, W) or not out.is_contiguous() or ctx.n_tokens != n or stride < W:
-        raise KernelError("lru_scan: y must be the step's float32 rows, out contiguous of the same shape, and the slot must hold a row")
-    for t, what in ((decay, "decay"), (gated, "gated")):
-        _dev(t, what)
-        if t.dtype != torch.float32 or tuple(t.shape) != (n, W) or not t.is_contiguous():
-            raise KernelError(f"lru_scan: {what} must be contiguous float32 [{n}, {W}]")
+    if y.dtype != torch.float32 or x.dtype != torch.float32 or tuple(x.shape) != (n, C) or tuple(out.shape) != (n, C) or not out.is_contiguous() or ctx.n_tokens != n:
+        raise KernelError("lru_scan: y and x must be the step's float32 rows and out contiguous of the same shape")
+    if z.dtype != torch.float32 or tuple(z.shape) != (n, 2 * C) or u.dtype != torch.float32 or tuple(u.shape) != (n, C) or not u.is_contiguous():
+        raise KernelError(f"lru_scan: z must be float32 rows [{n}, {2 * C}] and u contiguous float32 [{n}, {C}]")
+    if blocks < 1 or C % blocks or taps < 1 or stride < taps * C:
+        raise KernelError(f"lru_scan: {C} channels in {blocks} parts, {taps} taps, a slot of {stride} floats")
+    _f32vec(br, "br", C)
+    _f32vec(bi, "bi", C)
+    _f32vec(lam, "lam", C)
     _step_lists(ctx, n)
-    _lib.call("liyab_lru_scan", out.data_ptr(), dtype_code(out.dtype), decay.data_ptr(), gated.data_ptr(), y.data_ptr(), ldy, state.data_ptr(), stride,
-              state.shape[0], ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, W, _stream())
+    decay = gated = None
+    stretches = lru_stretches(ctx, n)
+    if stretches:
+        decay = ctx.workspace.get("lru_decay", (n, C), torch.float32)
+        gated = ctx.workspace.get("lru_gated", (n, C), torch.float32)
+        _lib.call("liyab_lru_coeffs", decay.data_ptr(), gated.data_ptr(), z.data_ptr(), ldz, u.data_ptr(), br.data_ptr(), bi.data_ptr(), lam.data_ptr(),
+                  float(rate), n, C, int(blocks), _stream())
+    _lib.call("liyab_lru_scan", out.data_ptr(), dtype_code(out.dtype), z.data_ptr(), ldz, u.data_ptr(), _ptr(decay), _ptr(gated), br.data_ptr(), bi.data_ptr(),
+              lam.data_ptr(), float(rate), float(out_scale), y.data_ptr(), ldy, state.data_ptr(), stride, state.shape[0], x.data_ptr(), ldx, int(taps),
+              ctx.seq_starts.data_ptr(), ctx.positions.data_ptr(), ctx.state_slots.data_ptr(), ctx.n_seqs, C, int(blocks), 1 if stretches else 0, _stream())

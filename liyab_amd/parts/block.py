@@ -236,11 +236,18 @@ class SandwichBlock:
         h = self.norm_mixer.forward(x, ctx, name="block_in")
         y = ws.get("sublayer_out", (n, d), torch.float32)
         self.mixer.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=y)
-        ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps)
+        # the update of the rows also takes the feed-forward's own norm of the new rows, where that is a root-mean-square norm too
+        fused = self.ffn is not None and getattr(self.norm_ffn, "root_mean_square", False) and self.norm_ffn.weight is not None
+        if fused:
+            h = ws.get("block_in", (n, d), self.norm_ffn.dtype)
+            ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps, cast_out=h, next_norm=(self.norm_ffn.weight, self.norm_ffn.eps))
+        else:
+            ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps)
         if self.ffn is not None:
             if ctx.phases is not None:
                 ctx.phases.mark(self.ffn_phase)
-            h = self.norm_ffn.forward(x, ctx, name="block_in")
+            if not fused:
+                h = self.norm_ffn.forward(x, ctx, name="block_in")
             k = int(getattr(self.ffn, "rows_a_token", 1))
             y = ws.get("sublayer_rows", (n * k, d), torch.float32) if k > 1 else y
             self.ffn.forward(h, ctx, None, out=y)

@@ -170,8 +170,14 @@ class ScoredAttention:
     def state_spec(self):
         return None
 
+    @property
+    def can_scale_output(self) -> bool:
+        """Whether forward(..., out_scale=, add=) is taken: the factor rides on the gate's pass over the heads' rows."""
+        return self.gated and (self.head_dim == self.value_dim or bool(self.row_dim))
+
     def forward(self, h, ctx: StepContext, cache: LayerCache, state, residual: Optional[torch.Tensor],
-                writes_cache: bool = True, out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None):
+                writes_cache: bool = True, out: Optional[torch.Tensor] = None, proj: Optional[torch.Tensor] = None,
+                out_scale: float = 1.0, add: bool = False):
         """Adds the mixer's result into `residual`, or, with `out` (float32 [n, width]), leaves it there. `proj`: the input
         projection's 32-bit rows (biases added, `in_bias`), when the caller has made them (as columns of a wider product)."""
         n, ws, H, D, V = h.shape[0], ctx.workspace, self.n_head, self.head_dim, self.value_dim
@@ -196,11 +202,17 @@ class ScoredAttention:
                                    softcap=self.softcap, bias_table=self.bias_table, sinks=self.sinks)
             assert splits is None
             if gate is not None:
-                ops.gate_rows(att, gate)
+                ops.gate_rows(att, gate, out_scale)
+            elif out_scale != 1.0:
+                raise Unsupported("scored attention: a factor on the result needs the gate's pass (can_scale_output)")
         else:
+            if out_scale != 1.0:
+                raise Unsupported("scored attention: a factor on the result needs the gate's pass (can_scale_output)")
             ops.attention_scored(att, q, cache.k, cache.v, group.block_tables, ctx, n_head=H, scale=self.scale, softcap=self.softcap,
                                  window=self.window, bias_table=self.bias_table, gate=gate, sinks=self.sinks)
-        if out is not None:
+        if out is not None and add:
+            linear(att, self.out_weight, None, residual=out)
+        elif out is not None:
             linear(att, self.out_weight, None, out=out)
         else:
             linear(att, self.out_weight, None, residual=settled(residual))

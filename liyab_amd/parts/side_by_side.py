@@ -70,6 +70,20 @@ class SideBySide:
     def forward(self, h, ctx: StepContext, cache, state, residual: Optional[torch.Tensor], writes_cache: bool = True,
                 out: Optional[torch.Tensor] = None):
         n, ws = h.shape[0], ctx.workspace
+        if not self.normed and all(getattr(p, "can_scale_output", False) for p in (self.left, self.right)):
+            # constant weights on results that are not normed: each mixer takes its factor where it rounds its rows for its last
+            # product, the first writes the sum's place and the second adds to it
+            y = out if out is not None else ws.get("side_left", (n, self.width), torch.float32)
+            proj_l = proj_r = None
+            if self.joint_weight is not None:
+                proj = ws.get("side_in", (n, self.joint_weight.shape[0]), torch.float32)
+                linear(h, self.joint_weight, self.joint_bias, out=proj)
+                proj_l, proj_r = proj[:, :self.left_cols], proj[:, self.left_cols:]
+            self.left.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=y, proj=proj_l, out_scale=self.left_weight)
+            self.right.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=y, proj=proj_r, out_scale=self.right_weight, add=True)
+            if out is None:
+                ops.add_into_(settled(residual), y)
+            return None
         a = ws.get("side_left", (n, self.width), torch.float32)
         b = ws.get("side_right", (n, self.width), torch.float32)
         if self.joint_weight is not None:
