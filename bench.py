@@ -6,7 +6,7 @@
     python bench.py --workload medium16|xl64         # the continuous-batching and the batch-64 workloads of the larger sizes
     python bench.py --link-floor                     # what one dependent kernel of a replayed graph costs at least
     python bench.py --product 4096,4096,16384,8,15   # one product in tiles of 128 x 128 and of 256 x 256
-    python bench.py --design bokulix|mofulix|dopilorn [--design-sizes small,medium,xl] [--layers L] [--phases]   # that design beside GPT-2 (dopilorn: beside Mofulix) at equal sizes
+    python bench.py --design bokulix|mofulix|dopilorn|larulorn [--design-sizes small,medium,xl] [--layers L] [--phases]   # that design beside GPT-2 (dopilorn, larulorn: beside Mofulix) at equal sizes
 
 The default run has GPT-2 small's layer sizes (12 layers, width 768, 12 heads
 of 64, feed-forward 3072, vocabulary 50257, 1024 positions) with random
@@ -566,10 +566,87 @@ def dopilorn_prefill_flops(cfg, prompt_lens, logit_rows):
     return flops
 
 
+# -- Larulorn beside Mofulix at equal sizes -------------------------------------------------------------------
+# The Larulorn of each size has GPT-2's width, layers, vocabulary and head count (heads of 64 everywhere); its layers take turns as
+# attention with a sink and biases (as many key heads as query heads, turned halves on a ramp, values mixed with the first layer's)
+# over a clamped feed-forward as Mofulix's, gated attention beside a gated linear recurrence as wide as the model (a part a head, four
+# taps) over the same feed-forward, and attention again over eight experts of a quarter of GPT-2's inner width in four groups of which
+# two stay, two experts a token, beside a shared expert of that width. It stands beside Mofulix, the engine's other design that mixes
+# recurrences with attention under a clamped feed-forward.
+def larulorn_config(gpt2_cfg):
+    d, H, F, L = gpt2_cfg["n_embd"], gpt2_cfg["n_head"], gpt2_cfg["n_inner"], gpt2_cfg["n_layer"]
+    hd = d // H
+    ff = max(64, F * 2 // 3 // 64 * 64)
+    dense = {"kind": "dense", "ff": ff, "limit": 7.0}
+    moe = {"kind": "moe", "expert": {"ff": F // 4}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": F // 4}}
+    rot = {"dims": hd, "base": 10000.0, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    own = {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": rot, "v_mix": True}
+    kinds = [
+        {"type": "attention", "mixer": own, "mlp": dense},
+        {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": {"dims": hd, "base": 10000.0}},
+                                       "right": {"width": d, "blocks": H, "conv": 4}, "left_scale": 0.8, "right_scale": 1.1}, "mlp": dense},
+        {"type": "attention", "mixer": own, "mlp": moe},
+    ]
+    return {"architecture": "Larulorn", "vocab": gpt2_cfg["vocab_size"], "width": d, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+            "max_positions": gpt2_cfg["n_positions"], "layers": [json.loads(json.dumps(kinds[i % 3])) for i in range(L)]}
+
+
+def _larulorn_layer_weights(entry, d, per_token=True):
+    """Matrix elements of a layer that a token's products read (2 flops an element a token); with `per_token` False, those a decode
+    step of many requests reads at most (every expert)."""
+    m, mlp = entry["mixer"], entry.get("mlp")
+    n = 0
+    if mlp and mlp["kind"] == "dense":
+        n += 3 * mlp["ff"] * d
+    elif mlp:
+        r = mlp["router"]
+        n += r["experts"] * d + (r["top"] if per_token else r["experts"]) * 2 * mlp["expert"]["ff"] * d + 2 * (mlp.get("shared") or {"ff": 0})["ff"] * d
+    a = m if entry["type"] == "attention" else m["left"]
+    n += (a["heads"] * a["dim"] + a["kv_heads"] * (a["dim"] + a["vdim"])) * d + d * a["heads"] * a["vdim"]
+    if entry["type"] == "parallel":
+        W, B = m["right"]["width"], m["right"]["blocks"]
+        n += a["heads"] * a["vdim"] * d + 3 * W * d + 2 * W * (W // B)
+    return n
+
+
+def larulorn_step_bytes(cfg, batch):
+    """The bytes a decode step has to read: every matrix a token of the batch can take (min(batch * top, experts) experts), the head, the
+    cached keys and values, and the 32-bit state of the recurrent layers (read and written) a request."""
+    def step_bytes(contexts, steps, elt):
+        d, V = cfg["width"], cfg["vocab"]
+        total = V * d * elt
+        seen = sum(sum(c + s + 1 for s in range(steps)) for c in contexts) / max(steps, 1)
+        for entry in cfg["layers"]:
+            m, mlp = entry["mixer"], entry.get("mlp")
+            n = _larulorn_layer_weights(entry, d, per_token=True)
+            if mlp and mlp["kind"] == "moe":
+                r = mlp["router"]
+                n += (min(len(contexts) * r["top"], r["experts"]) - r["top"]) * 2 * mlp["expert"]["ff"] * d
+            total += n * elt
+            a = m if entry["type"] == "attention" else m["left"]
+            total += seen * a["kv_heads"] * (a["dim"] + a["vdim"]) * elt
+            if entry["type"] == "parallel":
+                total += len(contexts) * 2 * m["right"]["width"] * m["right"]["conv"] * 4
+        return total
+    return step_bytes
+
+
+def larulorn_prefill_flops(cfg, prompt_lens, logit_rows):
+    d, V, n = cfg["width"], cfg["vocab"], sum(prompt_lens)
+    flops = 2.0 * logit_rows * d * V
+    pairs = sum(t * (t + 1) / 2 for t in prompt_lens)
+    for entry in cfg["layers"]:
+        m = entry["mixer"]
+        a = m if entry["type"] == "attention" else m["left"]
+        flops += 2.0 * n * _larulorn_layer_weights(entry, d) + 2.0 * pairs * a["heads"] * (a["dim"] + a["vdim"])
+    return flops
+
+
 DESIGNS = {"bokulix": (lambda gpt2, size: bokulix_config(gpt2, BOKULIX_SHAPES[size]), bokulix_step_bytes, bokulix_prefill_flops),
            "mofulix": (lambda gpt2, size: mofulix_config(gpt2), mofulix_step_bytes, mofulix_prefill_flops),
-           "dopilorn": (lambda gpt2, size: dopilorn_config(gpt2), dopilorn_step_bytes, dopilorn_prefill_flops)}
-BESIDE = {"dopilorn": "mofulix"}  # the engine's closest model, where that is not GPT-2
+           "dopilorn": (lambda gpt2, size: dopilorn_config(gpt2), dopilorn_step_bytes, dopilorn_prefill_flops),
+           "larulorn": (lambda gpt2, size: larulorn_config(gpt2), larulorn_step_bytes, larulorn_prefill_flops)}
+BESIDE = {"dopilorn": "mofulix", "larulorn": "mofulix"}  # the engine's closest model, where that is not GPT-2
 
 
 def design_run(args):
@@ -647,9 +724,9 @@ def main():
     ap.add_argument("--link-floor", action="store_true", help="measure what one dependent kernel of a replayed graph costs at least")
     ap.add_argument("--phases", action="store_true", help="device milliseconds per phase of the forward pass (embed, attention, dense_ffn, lm_head) a decode step "
                     "and a prefill of 2,048 tokens, as the reference's command line prints them (tools/liyab_cli.cpp:198-211); steps run kernel by kernel, without graphs")
-    ap.add_argument("--design", default="", choices=["", "bokulix", "mofulix", "dopilorn"],
+    ap.add_argument("--design", default="", choices=["", "bokulix", "mofulix", "dopilorn", "larulorn"],
                     help="bokulix, mofulix: that design beside GPT-2 at equal layer sizes (prefill and decode, both with their rooflines); "
-                         "dopilorn: beside Mofulix, the engine's closest model")
+                         "dopilorn, larulorn: beside Mofulix, the engine's closest model")
     ap.add_argument("--design-only", action="store_true", help="with --design: skip the GPT-2 run (for profiling)")
     ap.add_argument("--design-sizes", default="small,medium,xl", help="the sizes --design runs (of small, medium, xl)")
     args = ap.parse_args()

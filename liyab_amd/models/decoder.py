@@ -141,6 +141,12 @@ class DecoderModel:
         self.final_norm = build_part("norm", plan.final_norm, store, dtype) if plan.final_norm is not None else None
         self.head = build_part("head", plan.head, store, dtype)
         self.order = list(plan.order)
+        # a block may take the first norm of the block that follows it into its own last update of the rows (`chain_norm`): offered
+        # where the order runs every layer once, on its own cache, with nothing done to the stream between the two
+        if [e.layer for e in self.order] == list(range(len(self.blocks))) and all(e.cache_of is None and e.writes_cache for e in self.order):
+            for i in range(len(self.blocks) - 1):
+                if hasattr(self.blocks[i], "chain_norm") and (i + 1) not in self.entries:
+                    self.blocks[i].chain_norm(self.blocks[i + 1])
         # the parts' step planners, one of each name (every attention layer shares attention's)
         self.step_planners = []
         for block in self.blocks:

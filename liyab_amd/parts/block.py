@@ -215,7 +215,19 @@ class SandwichBlock:
     takes_padding_rows = True
     takes_pending = False
 
+    def chain_norm(self, following) -> bool:
+        """Called once, when the model is built, for a block that runs right before `following` in every pass: this block's last
+        update of the rows then also takes `following`'s first norm of them, and `following` reads those rows instead of taking its
+        norm itself. True if the two were chained (both sandwich blocks whose first norms are weighted root-mean-square norms)."""
+        norm = getattr(following, "norm_mixer", None)
+        if not isinstance(following, SandwichBlock) or not getattr(norm, "root_mean_square", False) or norm.weight is None or norm.dtype != self.norm_mixer.dtype:
+            return False
+        self.next_weight, self.next_eps = norm.weight, float(norm.eps)
+        following.input_normed = True
+        return True
+
     def __init__(self, spec, mixer, ffn, norm_mixer, norm_ffn, post_norm_mixer=None, post_norm_ffn=None):
+        self.next_weight, self.next_eps, self.input_normed = None, 0.0, False
         self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn if ffn is not None else None
         self.post_norm_mixer, self.post_norm_ffn = post_norm_mixer, post_norm_ffn if ffn is not None else None
         self.mixer_phase = getattr(getattr(spec, "mixer", None), "kind", "mixer")
@@ -233,14 +245,19 @@ class SandwichBlock:
         ws, n, d = ctx.workspace, x.shape[0], x.shape[1]
         if ctx.phases is not None:
             ctx.phases.mark(self.mixer_phase)
-        h = self.norm_mixer.forward(x, ctx, name="block_in")
+        # (the block before may have left this block's first norm of the rows where this block's own norm would put it)
+        h = ws.get("block_in", (n, d), self.norm_mixer.dtype) if self.input_normed else self.norm_mixer.forward(x, ctx, name="block_in")
         y = ws.get("sublayer_out", (n, d), torch.float32)
         self.mixer.forward(h, ctx, cache, state, None, writes_cache=writes_cache, out=y)
-        # the update of the rows also takes the feed-forward's own norm of the new rows, where that is a root-mean-square norm too
+        # the update of the rows also takes the next norm of the new rows, where that is a root-mean-square norm too: the feed-forward's
+        # own, or, behind the layer's last sublayer, the next layer's first
+        chained = (self.next_weight, self.next_eps) if self.next_weight is not None else None
         fused = self.ffn is not None and getattr(self.norm_ffn, "root_mean_square", False) and self.norm_ffn.weight is not None
         if fused:
             h = ws.get("block_in", (n, d), self.norm_ffn.dtype)
             ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps, cast_out=h, next_norm=(self.norm_ffn.weight, self.norm_ffn.eps))
+        elif self.ffn is None and chained is not None:
+            ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps, cast_out=ws.get("block_in", (n, d), self.norm_mixer.dtype), next_norm=chained)
         else:
             ops.gated_norm_add(x, y, self.post_norm_mixer.weight, self.post_norm_mixer.eps)
         if self.ffn is not None:
@@ -251,7 +268,11 @@ class SandwichBlock:
             k = int(getattr(self.ffn, "rows_a_token", 1))
             y = ws.get("sublayer_rows", (n * k, d), torch.float32) if k > 1 else y
             self.ffn.forward(h, ctx, None, out=y)
-            ops.gated_norm_add(x, y, self.post_norm_ffn.weight, self.post_norm_ffn.eps, n_sum=k)
+            if chained is not None:
+                ops.gated_norm_add(x, y, self.post_norm_ffn.weight, self.post_norm_ffn.eps, n_sum=k, cast_out=ws.get("block_in", (n, d), self.norm_mixer.dtype),
+                                   next_norm=chained)
+            else:
+                ops.gated_norm_add(x, y, self.post_norm_ffn.weight, self.post_norm_ffn.eps, n_sum=k)
         return None
 
 

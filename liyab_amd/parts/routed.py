@@ -44,7 +44,7 @@ class RoutedFFN:
         self.gate = store.fetch_joined([t[("gate", e)] for e in range(E)], [(F, d)] * E, "matrix", "stack") if self.gated else None
         self.up = store.fetch_joined([t[("up", e)] for e in range(E)], [(F, d)] * E, "matrix", "stack")
         self.down = store.fetch_joined([t[("down", e)] for e in range(E)], [(d, F)] * E, "matrix", "stack")
-        self.shared_in = self.shared_down = None
+        self.shared_in = self.shared_down = self.joint_in = None
         if self.shared_inner:
             if self.gated:
                 raise Unsupported("routed feed-forward: a shared expert beside gated experts is not supported")
@@ -52,13 +52,17 @@ class RoutedFFN:
             names = ([t["shared_gate"]] if self.gated else []) + [t["shared_up"]]
             self.shared_in = store.fetch_joined(names, [(S, d)] * len(names), "matrix", "rows")
             self.shared_down = store.fetch(t["shared_down"], (d, S), "matrix")
+            # the router and the shared expert's first product read the same rows: one product [router | shared]
+            if self.router_bias is None and self.router.dtype == self.shared_in.dtype:
+                rw, sw = self.router, self.shared_in
+                self.joint_in = store.derived(("joined_rows", t["router"].name, t["shared_up"].name), lambda: torch.cat([rw, sw], dim=0).contiguous())
 
     def take_router(self):
         """(weight [experts, width], bias or None): the router's product handed to a caller that runs it as rows
         of a wider product over the same input and passes the logits to `forward(..., router_logits=)`; this
         part then no longer holds the matrix."""
         w, b = self.router, self.router_bias
-        self.router = self.router_bias = None
+        self.router = self.router_bias = self.joint_in = None
         return w, b
 
     rows_a_token = property(lambda self: self.top + (1 if self.shared_inner else 0))  # rows `forward(..., out=)` leaves for each token
@@ -71,7 +75,11 @@ class RoutedFFN:
         has computed them already, beside a product of its own over the same rows (`take_router`)."""
         h = as_tensor(h)
         n, ws, E, top = h.shape[0], ctx.workspace, self.n_experts, self.top
-        logits = router_logits
+        logits, shared_pre = router_logits, None
+        if logits is None and self.joint_in is not None:
+            z = ws.get("router_shared", (n, self.joint_in.shape[0]), torch.float32)
+            linear(h, self.joint_in, None, out=z)
+            logits, shared_pre = z[:, :E], z[:, E:]
         if logits is None:
             logits = ws.get("router_logits", (n, E), torch.float32)
             linear(h, self.router, self.router_bias, out=logits)
@@ -93,10 +101,11 @@ class RoutedFFN:
         ops.moe_product(y, inner, self.down, None, rows_list, tile_group, row_scale=weights, block=block, out_div=top, out_extra=rows - top)
         if self.shared_inner:
             S = self.shared_inner
-            z = ws.get("shared_in", (n, self.shared_in.shape[0]), torch.float32)
-            linear(h, self.shared_in, None, out=z)
+            if shared_pre is None:
+                shared_pre = ws.get("shared_in", (n, self.shared_in.shape[0]), torch.float32)
+                linear(h, self.shared_in, None, out=shared_pre)
             act = ws.get("shared_inner", (n, S), self.dtype)
-            ops.activate(act, z, self.activation)
+            ops.activate(act, shared_pre, self.activation)
             # the shared expert's row of each token, behind its `top` rows
             linear(act, self.shared_down, None, out=y.view(n, rows * self.width)[:, top * self.width:])
         if out is None:
