@@ -24,17 +24,20 @@ DTYPES = ["float32", "bfloat16"]
 # float32: the largest difference of a row relative to its largest |logit|, as for the other models.
 # bfloat16, against the twin in float64 with the same rounded matrices: the root mean square of a row's difference over
 # that of the row's logits, both with their means taken off; a fault in a mechanism makes it about 1.
-# Every sublayer's result passes a norm before it joins the stream, which brings each rounding back to the stream's own
-# size, layer after layer: the three larger geometries show 0.02 to 0.03, the drawn ones up to 0.08.
-TOL_B = {"float32": TOL["float32"], "bfloat16": 2e-1}
+# The five geometries and the wide model show 0.01 to 0.03. Among the drawn geometries a row here and there reaches 0.13 (the
+# row's 99th percentile stays below 0.04): every sublayer's result passes a norm before it joins the stream, which brings each
+# rounding back to the stream's own size, layer after layer, and a drawn scale may leave a softmax closely contested.
+TOL_B = {"float32": TOL["float32"], "bfloat16": 6e-2}
+TOL_DRAWN = 2e-1
 KEPT_32BIT = (".conv", ".ra.b", ".ri.b")  # 2-D tensors that the engine keeps in 32 bits
 ROUNDED_3D = (".ra", ".ri")  # the recurrence's gates, a matrix a part
 
 
-def check_logits(got, reqs, ref, dtype, what, family=None):
+def check_logits(got, reqs, ref, dtype, what, family=None, tol=None):
     if dtype == "float32":
         return tt.check_against_plain(got, reqs, ref, TOL_B[dtype], what, family=family)
-    key = ((family or what.split(" ")[0]) + " (rms)", TOL_B[dtype])
+    tol = tol or TOL_B[dtype]
+    key = ((family or what.split(" ")[0]) + " (rms)", tol)
     for rid, toks in reqs.items():
         assert rid in got, f"{what}: no logits for request {rid}"
         for p in sorted(got[rid]):
@@ -43,7 +46,7 @@ def check_logits(got, reqs, ref, dtype, what, family=None):
             diff = row - want
             e = float(np.sqrt(np.mean((diff - diff.mean()) ** 2)) / np.sqrt(np.mean((want - want.mean()) ** 2)))
             tt.WORST[key] = max(tt.WORST.get(key, 0.0), e)
-            assert e <= TOL_B[dtype], f"{what}: request {rid} (length {len(toks)}) first differs at position {p}: {e:.3e} > {TOL_B[dtype]:.1e}"
+            assert e <= tol, f"{what}: request {rid} (length {len(toks)}) first differs at position {p}: {e:.3e} > {tol:.1e}"
 
 
 # ---------------------------------------------------------------------------
@@ -643,10 +646,10 @@ def test_drawn_geometries_whole_and_mixed(seed, tmp_path):
         ref = {rid: plain.forward(raw, t, toks) for rid, toks in reqs.items()}
         steps = tt.schedule_whole(reqs)
         core = make_core(d, dtype, tt.max_live_tokens(steps), page_size=page_size)
-        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"larulorn-drawn seed {seed} whole {dtype}", family="larulorn-drawn")
+        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"larulorn-drawn seed {seed} whole {dtype}", family="larulorn-drawn", tol=TOL_DRAWN)
         steps = tt.schedule_mixed(reqs, seed=seed, max_live=3)
         core = make_core(d, dtype, None, page_size=page_size, max_requests=3, num_pages=tt.max_live_pages(steps, page_size))
-        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"larulorn-drawn seed {seed} mixed {dtype}", family="larulorn-drawn")
+        check_logits(tt.run_schedule(core, steps), reqs, ref, dtype, f"larulorn-drawn seed {seed} mixed {dtype}", family="larulorn-drawn", tol=TOL_DRAWN)
         core.manager.check()
 
 
