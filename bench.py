@@ -584,7 +584,7 @@ def larulorn_config(gpt2_cfg):
     kinds = [
         {"type": "attention", "mixer": own, "mlp": dense},
         {"type": "parallel", "mixer": {"left": {"heads": H, "kv_heads": H, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "rot": {"dims": hd, "base": 10000.0}},
-                                       "right": {"width": d, "blocks": H, "conv": 4}, "left_scale": 0.8, "right_scale": 1.1}, "mlp": dense},
+                                       "right": {"width": d, "blocks": H, "conv": 4}, "left_scale": 0.75, "right_scale": 1.25}, "mlp": dense},
         {"type": "attention", "mixer": own, "mlp": moe},
     ]
     return {"architecture": "Larulorn", "vocab": gpt2_cfg["vocab_size"], "width": d, "norm": {"eps": 1e-5}, "logit_scale": 1.0,
