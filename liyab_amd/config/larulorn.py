@@ -129,11 +129,13 @@ def _attention(m, where: str, mixes: bool) -> LarulornAttention:
     dims, base, ramp = 0, 0.0, None
     if rot is not None:
         dims, base = _int(rot, "dims", where + ".rot.dims"), _number(rot, "base", where + ".rot.base")
-        if dims % 2 or dims > D or base == 1.0:
-            raise InvalidModel(f"invalid {where}.rot: {dims} turned entries of heads of {D}, base {base}")
+        if dims % 2 or dims > D:
+            raise InvalidModel(f"invalid {where}.rot: {dims} turned entries of heads of {D}")
         sc = rot.get("scaling") if isinstance(rot, dict) else None
         if sc is not None:
             ramp = tuple(_number(sc, k, f"{where}.rot.scaling.{k}") for k in ("factor", "fast", "slow", "original"))
+            if base == 1.0:
+                raise InvalidModel(f"invalid {where}.rot: a ramp over the entries needs a base other than one")
     v_mix = m.get("v_mix", False)
     if not isinstance(v_mix, bool) or (v_mix and not mixes):
         raise InvalidModel(f"invalid {where}.v_mix")
